@@ -1,0 +1,170 @@
+"""The flat batch of one step.
+
+The reference's forward takes a padded [B, S] token matrix that is either all
+prompts of one length or all single tokens, plus a shared mutable AttentionInfo
+(lite_llama/executor/model_executor.py:314-320, lite_llama/executor/
+executor_struct.py:12-17). Here a step is a list of (request, its next tokens,
+the places whose logits are wanted), cut anywhere, and everything a kernel
+needs travels in one StepContext.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import torch
+
+ATTN_BLOCK_ROWS = 16    # query rows per work item of the attention kernels
+
+
+@dataclass
+class StepEntry:
+    """The next tokens of one request and the indices among them whose logits
+    are wanted (``want`` may be empty)."""
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class GroupContext:
+    block_table: torch.Tensor      # int32 [n, max_pages]; row i = sequence i of the batch
+    slots: torch.Tensor            # int32 [T]: cache slot of every token of the batch
+
+
+@dataclass
+class StepContext:
+    token_ids: torch.Tensor        # int32 [T]
+    positions: torch.Tensor        # int32 [T]
+    q_start: torch.Tensor          # int32 [n+1]: first row of every sequence
+    ctx_len: torch.Tensor          # int32 [n]: tokens of the sequence in the cache after this step
+    state_slots: torch.Tensor      # int32 [n]: state slot of every sequence
+    logit_rows: torch.Tensor       # int32 [R]: rows whose logits are wanted
+    work_seq: torch.Tensor         # int32 [W]: attention work items (sequence,
+    work_qoff: torch.Tensor        # int32 [W]:   first query row within it)
+    groups: List[GroupContext]
+    num_tokens: int
+    num_seqs: int
+    num_logit_rows: int
+    logit_rows_are_identity: bool
+    num_decode_seqs: int           # leading sequences that bring a single token
+    q_lens: List[int] = field(default_factory=list)       # host copies
+    ctx_lens: List[int] = field(default_factory=list)
+    max_q_len: int = 0
+    max_ctx_len: int = 0
+
+
+def order_entries(entries: Sequence[StepEntry]) -> List[int]:
+    """Single-token entries first (stable), so that kernels specialised for the
+    decode case see one contiguous range of sequences."""
+    idx = list(range(len(entries)))
+    return [i for i in idx if len(entries[i].tokens) == 1] + \
+           [i for i in idx if len(entries[i].tokens) != 1]
+
+
+def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Optional[int] = None):
+    """Take pages for every entry (all or nothing) and lay the batch out.
+    Returns (StepContext, order) where ``order`` is the permutation applied to
+    the entries; logit rows are listed in the caller's order of entries."""
+    if not entries:
+        raise ValueError("a step needs at least one entry")
+    seen = set()
+    for e in entries:
+        if len(e.tokens) == 0:
+            raise ValueError(f"request {e.request!r} brings no tokens")
+        if e.request in seen:
+            raise ValueError(f"request {e.request!r} appears twice in one step")
+        seen.add(e.request)
+        for w in e.want:
+            if not 0 <= w < len(e.tokens):
+                raise ValueError(f"request {e.request!r}: wanted place {w} outside its "
+                                 f"{len(e.tokens)} tokens")
+        if vocab_size is not None:
+            for t in e.tokens:
+                if not 0 <= t < vocab_size:
+                    raise ValueError(f"request {e.request!r}: token id {t} outside the "
+                                     f"vocabulary of {vocab_size}")
+    # pages: check the whole step before taking anything
+    need = [0] * len(manager.paged)
+    for e in entries:
+        for g, n in enumerate(manager.pages_needed(e.request, len(e.tokens))):
+            need[g] += n
+    for g, n in enumerate(need):
+        if n > manager.paged[g].pool.num_free:
+            from ..cache.manager import OutOfPages
+            raise OutOfPages(f"the step needs {n} pages of group {g}, "
+                             f"{manager.paged[g].pool.num_free} are free")
+
+    order = order_entries(entries)
+    token_ids: List[int] = []
+    positions: List[int] = []
+    q_start = [0]
+    ctx_len: List[int] = []
+    state_slots: List[int] = []
+    slots: List[List[int]] = [[] for _ in manager.paged]
+    row_of_entry = {}
+    for i in order:
+        e = entries[i]
+        n = len(e.tokens)
+        start = manager.append(e.request, n)
+        row_of_entry[i] = q_start[-1]
+        token_ids.extend(int(t) for t in e.tokens)
+        positions.extend(range(start, start + n))
+        q_start.append(q_start[-1] + n)
+        ctx_len.append(start + n)
+        state_slots.append(manager.slot_of[e.request])
+        for g in range(len(manager.paged)):
+            slots[g].extend(manager.slots(e.request, g, start, n))
+    logit_rows = [row_of_entry[i] + w for i, e in enumerate(entries) for w in e.want]
+    T = len(token_ids)
+    nseq = len(order)
+    q_lens = [q_start[i + 1] - q_start[i] for i in range(nseq)]
+    work_seq, work_qoff = [], []
+    for s, ql in enumerate(q_lens):
+        for off in range(0, ql, ATTN_BLOCK_ROWS):
+            work_seq.append(s)
+            work_qoff.append(off)
+    tables = []
+    for g, group in enumerate(manager.paged):
+        rows = [group.tables[entries[i].request] for i in order]
+        width = max(1, max(len(r) for r in rows))
+        tables.append([r + [-1] * (width - len(r)) for r in rows])
+
+    # one host->device copy for all integer arrays
+    flat: List[int] = []
+    spans = {}
+
+    def put(name, values):
+        spans[name] = (len(flat), len(values))
+        flat.extend(values)
+
+    put("token_ids", token_ids)
+    put("positions", positions)
+    put("q_start", q_start)
+    put("ctx_len", ctx_len)
+    put("state_slots", state_slots)
+    put("logit_rows", logit_rows)
+    put("work_seq", work_seq)
+    put("work_qoff", work_qoff)
+    for g in range(len(manager.paged)):
+        put(f"slots{g}", slots[g])
+        put(f"table{g}", [p for row in tables[g] for p in row])
+    buf = torch.tensor(flat, dtype=torch.int32)
+    if torch.device(device).type != "cpu":
+        buf = buf.pin_memory().to(device, non_blocking=True)
+
+    def get(name):
+        a, n = spans[name]
+        return buf[a:a + n]
+
+    groups = [GroupContext(get(f"table{g}").view(nseq, -1), get(f"slots{g}"))
+              for g in range(len(manager.paged))]
+    ctx = StepContext(
+        token_ids=get("token_ids"), positions=get("positions"), q_start=get("q_start"),
+        ctx_len=get("ctx_len"), state_slots=get("state_slots"), logit_rows=get("logit_rows"),
+        work_seq=get("work_seq"), work_qoff=get("work_qoff"), groups=groups,
+        num_tokens=T, num_seqs=nseq, num_logit_rows=len(logit_rows),
+        logit_rows_are_identity=logit_rows == list(range(T)),
+        num_decode_seqs=sum(1 for q in q_lens if q == 1),
+        q_lens=q_lens, ctx_lens=ctx_len, max_q_len=max(q_lens), max_ctx_len=max(ctx_len))
+    return ctx, order

@@ -1,0 +1,53 @@
+"""The step function: run a batch of (request, next tokens) through the model
+from the cache and return the logits at the wanted places."""
+from __future__ import annotations
+
+from typing import Hashable, List, Optional, Sequence
+
+import torch
+
+from .. import ops
+from ..cache import CacheManager, CacheStorage
+from .batch import StepEntry, build_context
+
+
+class ModelRunner:
+    """Owns the cache (bookkeeping and device memory) of one loaded model.
+
+    ``step`` runs only the tokens it is given, as one batch: portions of
+    prompts beside single decoded tokens, cut anywhere. A request is admitted
+    when it first appears and lives until ``end``. The reference's counterpart
+    is ModelExecutor.forward with prefill_alloc_kv_cache / decode_alloc_kv_cache
+    around it (lite_llama/executor/model_executor.py:261-320)."""
+
+    def __init__(self, model, page_size: int, num_pages, max_num_seqs: int):
+        if model.dtype is None:
+            raise RuntimeError("load the model's weights before making a runner")
+        self.model = model
+        self.device = model.device
+        if self.device.type == "cuda":
+            ops.library.require(model.kernel_libraries())
+        self.manager = CacheManager(model.cache_layers, page_size, num_pages, max_num_seqs)
+        self.storage = CacheStorage(self.manager, model.dtype, self.device)
+
+    def admit(self, request: Hashable) -> None:
+        slot = self.manager.admit(request)
+        self.storage.clear_slot(slot)
+
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Float32 logits [wanted, vocab], in the order of the entries and of
+        their ``want`` lists."""
+        for e in entries:
+            if not self.manager.is_live(e.request):
+                self.admit(e.request)
+        ctx, _ = build_context(entries, self.manager, self.device, self.model.vocab_size)
+        logits = self.model.forward(ctx, self.storage)
+        for e in entries:
+            self.manager.release_behind_window(e.request)
+        return logits
+
+    def end(self, request: Hashable) -> None:
+        """The request is finished: what it holds is given back."""
+        if self.manager.is_live(request):
+            self.manager.free(request)

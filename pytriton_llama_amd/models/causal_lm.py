@@ -1,0 +1,90 @@
+"""The container every architecture builds: embedding, blocks, final norm, head,
+the cache layers the blocks use and the order in which blocks run."""
+from __future__ import annotations
+
+import fnmatch
+from dataclasses import dataclass
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..parts.base import ParamSource, Part
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    """One entry of the run order: run ``block`` with cache layer
+    ``cache_layer`` (None: the block keeps nothing). ``writes`` False lets a
+    block read a cache layer that another call fills. A block, and a cache
+    layer, may be named by several calls."""
+    block: int
+    cache_layer: Optional[int]
+    writes: bool = True
+
+
+class CausalLM:
+    """A decoder-only language model as data: parts plus a run order.
+
+    ``prefixes`` maps every part to the checkpoint prefix of its tensors:
+    a list of (prefix, part). ``ignorable`` are glob patterns of checkpoint
+    tensors that may be present without being used."""
+
+    def __init__(self, config: Any, embedding: Part, blocks: Sequence[Part], final_norm: Part,
+                 head: Part, cache_layers: Sequence[object], schedule: Sequence[LayerCall],
+                 prefixes: Sequence[Tuple[str, Part]], ignorable: Sequence[str] = ()):
+        self.config = config
+        self.embedding, self.blocks = embedding, list(blocks)
+        self.final_norm, self.head = final_norm, head
+        self.cache_layers = list(cache_layers)
+        self.schedule = list(schedule)
+        self.prefixes = list(prefixes)
+        self.ignorable = tuple(ignorable)
+        for call in self.schedule:
+            if not 0 <= call.block < len(self.blocks):
+                raise ValueError(f"run order names block {call.block}, there are {len(self.blocks)}")
+            if call.cache_layer is not None and not 0 <= call.cache_layer < len(self.cache_layers):
+                raise ValueError(f"run order names cache layer {call.cache_layer}, "
+                                 f"there are {len(self.cache_layers)}")
+        self.dtype: Optional[torch.dtype] = None
+        self.device = None
+
+    # ---- what the loader and the builder need -------------------------------
+    def expected_tensors(self) -> Dict[str, Tuple[Part, ParamSource]]:
+        out: Dict[str, Tuple[Part, ParamSource]] = {}
+        for prefix, part in self.prefixes:
+            for src in part.param_sources():
+                name = prefix + src.name
+                if name in out:
+                    raise ValueError(f"two parts ask for checkpoint tensor {name!r}")
+                out[name] = (part, src)
+        return out
+
+    def is_ignorable(self, name: str) -> bool:
+        return any(fnmatch.fnmatchcase(name, pat) for pat in self.ignorable)
+
+    def kernel_libraries(self) -> Tuple[str, ...]:
+        libs: Tuple[str, ...] = ()
+        for part in [self.embedding, *self.blocks, self.final_norm, self.head]:
+            libs += tuple(part.kernel_libraries)
+        return tuple(dict.fromkeys(libs))
+
+    @property
+    def vocab_size(self) -> int:
+        return self.head.vocab_size
+
+    # ---- the forward pass of one step ------------------------------------------
+    def forward(self, ctx, storage) -> torch.Tensor:
+        """Float32 logits [len(ctx.logit_rows), vocab] for the flat batch ``ctx``."""
+        h = self.embedding.forward(ctx.token_ids)
+        residual = None
+        for call in self.schedule:
+            cache = storage.view(call.cache_layer, call.writes)
+            h, residual = self.blocks[call.block].forward(h, residual, ctx, cache)
+        if ctx.num_logit_rows == 0:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=h.device)
+        if ctx.num_logit_rows != h.shape[0] or not ctx.logit_rows_are_identity:
+            h = h.index_select(0, ctx.logit_rows)
+            if residual is not None:
+                residual = residual.index_select(0, ctx.logit_rows)
+        h, _ = self.final_norm.forward(h, residual)
+        return self.head.forward(h)

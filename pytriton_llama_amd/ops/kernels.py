@@ -1,0 +1,249 @@
+"""Python faces of the HIP kernels: each checks on the host that the operands
+match what the kernel and its grid assume (device, dtype, shape, strides) and
+then launches on torch's current stream. There is no CPU path and no library
+fallback: an operand that is not on the GPU, or a size a kernel does not take,
+raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library
+
+_F32, _BF16 = 0, 1
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return _F32
+    if t.dtype == torch.bfloat16:
+        return _BF16
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}")
+
+
+def _need_gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("HIP kernels need tensors on the GPU (there is no CPU path); "
+                              f"got a tensor on {t.device}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(code: int, what: str) -> None:
+    if code == 0:
+        return
+    if code == -1:
+        raise KernelError(f"{what}: the kernel refused these sizes or arguments")
+    raise KernelError(f"{what}: kernel launch failed (code {code})")
+
+
+def _i32(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{name} must be a contiguous int32 tensor")
+
+
+# ---------------------------------------------------------------------------
+def embedding(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[ids[t]]; ids int32 [T]."""
+    _need_gpu(table, ids)
+    _i32(ids, "ids")
+    if table.dim() != 2 or not table.is_contiguous():
+        raise KernelError("embedding table must be a contiguous [V, H] matrix")
+    V, H = table.shape
+    T = ids.numel()
+    out = torch.empty((T, H), dtype=table.dtype, device=table.device)
+    lib = library.load("embedding")
+    _check(lib.ptl_embedding(_ptr(out), _ptr(table), _ptr(ids), T, H, V, _dtype_code(table),
+                             _stream()), "embedding")
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor,
+                eps: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = rmsnorm(x + residual) * weight; ``residual`` (if given) is replaced
+    by the sum in place. weight is float32 [H]. Returns y."""
+    _need_gpu(x, residual, weight)
+    if x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("add_rmsnorm: x must be a contiguous [T, H] matrix")
+    T, H = x.shape
+    if weight.dtype != torch.float32 or weight.shape != (H,) or not weight.is_contiguous():
+        raise KernelError(f"add_rmsnorm: weight must be float32 [{H}]")
+    if residual is not None and (residual.shape != x.shape or residual.dtype != x.dtype
+                                 or not residual.is_contiguous()):
+        raise KernelError("add_rmsnorm: residual must match x in shape and dtype")
+    if H * 4 > 60000:
+        raise KernelError(f"add_rmsnorm: width {H} exceeds the kernel's limit of 15000")
+    y = out if out is not None else torch.empty_like(x)
+    lib = library.load("norm")
+    _check(lib.ptl_add_rmsnorm(_ptr(y), _ptr(x), _ptr(residual), _ptr(weight), T, H,
+                               ctypes.c_float(eps), _dtype_code(x), _stream()), "add_rmsnorm")
+    return y
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """out[:, i] = silu(gate_up[:, i]) * gate_up[:, I + i] for a [T, 2I] input."""
+    _need_gpu(gate_up)
+    if gate_up.dim() != 2 or not gate_up.is_contiguous() or gate_up.shape[1] % 2:
+        raise KernelError("silu_mul: input must be a contiguous [T, 2I] matrix")
+    T, I2 = gate_up.shape
+    out = torch.empty((T, I2 // 2), dtype=gate_up.dtype, device=gate_up.device)
+    lib = library.load("activation")
+    _check(lib.ptl_silu_mul(_ptr(out), _ptr(gate_up), T, I2 // 2, _dtype_code(gate_up), _stream()),
+           "silu_mul")
+    return out
+
+
+def rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor,
+               inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+               k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+               page_size: int = 1, k_in_place: bool = False) -> None:
+    """Rotate q in place (and k, when ``k_in_place``) by the angles
+    positions * inv_freq and write the rotated k and v into the caches
+    [num_pages, Hkv, page_size, D] at ``slots`` (int32, page*page_size+offset).
+    q, k, v are [T, heads, D] views that share one row stride (slices of one
+    projection output). inv_freq None: no rotation. slots None: no store."""
+    _need_gpu(q, k, v, positions, inv_freq, slots, k_cache, v_cache)
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    if k.shape != (T, Hkv, D) or v.shape != (T, Hkv, D):
+        raise KernelError("rope_store: k and v must be [T, Hkv, D]")
+    rs = q.stride(0)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if t.stride(2) != 1 or t.stride(1) != D or t.stride(0) != rs or t.dtype != q.dtype:
+            raise KernelError(f"rope_store: {name} must be a [T, heads, D] view with dense heads "
+                              "and the common row stride")
+    _i32(positions, "positions")
+    if positions.numel() != T:
+        raise KernelError("rope_store: one position per token")
+    if D % 2:
+        raise KernelError(f"rope_store: head size {D} must be even")
+    if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != D // 2
+                                 or not inv_freq.is_contiguous()):
+        raise KernelError(f"rope_store: inv_freq must be float32 [{D // 2}]")
+    if slots is not None:
+        if slots.dtype != torch.int32 or slots.numel() != T or not slots.is_contiguous():
+            raise KernelError("rope_store: slots must be contiguous int32 [T]")
+        for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+            if c is None or c.dim() != 4 or c.shape[1:] != (Hkv, page_size, D) \
+                    or c.dtype != q.dtype or not c.is_contiguous():
+                raise KernelError(f"rope_store: {name} must be contiguous "
+                                  f"[pages, {Hkv}, {page_size}, {D}] of {q.dtype}")
+    lib = library.load("rope")
+    _check(lib.ptl_rope_store(_ptr(q), _ptr(k), _ptr(v), ctypes.c_long(rs), _ptr(positions),
+                              _ptr(inv_freq), _ptr(slots), _ptr(k_cache), _ptr(v_cache),
+                              T, Hq, Hkv, D, page_size, int(k_in_place), _dtype_code(q),
+                              _stream()), "rope_store")
+
+
+def gemm_nt(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = x @ w.T with float32 accumulation through the vector-FMA kernel.
+    x [M, K] (rows may be strided), w [N, K] contiguous, same dtype."""
+    _need_gpu(x, w)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelError(f"gemm_nt: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
+    if x.dtype != w.dtype:
+        raise KernelError(f"gemm_nt: x is {x.dtype} but w is {w.dtype}")
+    if x.stride(1) != 1 or not w.is_contiguous():
+        raise KernelError("gemm_nt: x rows and w must be dense")
+    M, K = x.shape
+    N = w.shape[0]
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == torch.float32 and out_dtype != torch.float32:
+        raise KernelError("gemm_nt: float32 inputs give float32 outputs")
+    y = out if out is not None else torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if M == 0:
+        return y
+    lib = library.load("gemm")
+    _check(lib.ptl_gemm_nt(_ptr(y), _ptr(x), _ptr(w), M, N, K, ctypes.c_long(x.stride(0)),
+                           ctypes.c_long(y.stride(0)), _dtype_code(x),
+                           _F32 if out_dtype == torch.float32 else _BF16, _stream()), "gemm_nt")
+    return y
+
+
+def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                      v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
+                      block_table: torch.Tensor, work_seq: torch.Tensor, work_qoff: torch.Tensor,
+                      scale: float, window: int = 0) -> None:
+    """Attention of a mixed batch over the paged cache (see csrc/attention.hip).
+    q [T, Hq, D] (rows may be strided), out [T, Hq, D], caches
+    [pages, Hkv, page_size, D], q_start [n+1], ctx_len [n], block_table [n, max_pages],
+    work_seq / work_qoff: the list of 16-row query blocks."""
+    _need_gpu(out, q, k_cache, v_cache, q_start, ctx_len, block_table, work_seq, work_qoff)
+    T, Hq, D = q.shape
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[3] != D:
+        raise KernelError("attention: caches must be [pages, Hkv, page_size, D]")
+    Hkv, page_size = k_cache.shape[1], k_cache.shape[2]
+    if D > 256:
+        raise KernelError(f"attention: head size {D} exceeds the kernel's limit of 256")
+    if Hq % Hkv:
+        raise KernelError(f"attention: {Hq} query heads are not a multiple of {Hkv} kv heads")
+    if q.stride(2) != 1 or q.stride(1) != D or out.stride(2) != 1 or out.stride(1) != D:
+        raise KernelError("attention: q and out need dense heads")
+    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
+        raise KernelError("attention: q, out and the caches must share one dtype")
+    if not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("attention: caches must be contiguous")
+    for name, t in (("q_start", q_start), ("ctx_len", ctx_len), ("work_seq", work_seq),
+                    ("work_qoff", work_qoff)):
+        _i32(t, name)
+    n = ctx_len.numel()
+    if q_start.numel() != n + 1 or work_seq.numel() != work_qoff.numel():
+        raise KernelError("attention: inconsistent sequence tables")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.shape[0] < n \
+            or block_table.stride(1) != 1:
+        raise KernelError("attention: block_table must be int32 [n, max_pages]")
+    lib = library.load("attention")
+    _check(lib.ptl_attention_generic(
+        _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
+        _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
+        int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), int(work_seq.numel()),
+        Hq, Hkv, D, page_size, int(window), ctypes.c_float(scale), _dtype_code(q), _stream()),
+        "attention")
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """Greedy token per row of float32 logits [R, V]; ties go to the lowest id."""
+    _need_gpu(logits)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("argmax: logits must be float32 [R, V] with dense rows")
+    R, V = logits.shape
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    lib = library.load("sampling")
+    _check(lib.ptl_argmax(_ptr(out), _ptr(logits), R, V, ctypes.c_long(logits.stride(0)), _stream()),
+           "argmax")
+    return out
+
+
+def sample_top_p(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
+                 uniform: torch.Tensor, return_probs: bool = False):
+    """One token per row from the nucleus of softmax(logits / temperature).
+    temperature, top_p, uniform: float32 [R] on the GPU."""
+    _need_gpu(logits, temperature, top_p, uniform)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("sample_top_p: logits must be float32 [R, V] with dense rows")
+    R, V = logits.shape
+    for name, t in (("temperature", temperature), ("top_p", top_p), ("uniform", uniform)):
+        if t.dtype != torch.float32 or t.numel() != R or not t.is_contiguous():
+            raise KernelError(f"sample_top_p: {name} must be float32 [{R}]")
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    probs = torch.empty((R, V), dtype=torch.float32, device=logits.device) if return_probs else None
+    lib = library.load("sampling")
+    _check(lib.ptl_sample_top_p(_ptr(out), _ptr(probs), _ptr(logits), R, V,
+                                ctypes.c_long(logits.stride(0)), _ptr(temperature), _ptr(top_p),
+                                _ptr(uniform), _stream()), "sample_top_p")
+    return (out, probs) if return_probs else out

@@ -1,0 +1,89 @@
+"""The attention mixer over the paged cache."""
+from __future__ import annotations
+
+import math
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from .base import PagedKVSpec, ParamSource, Part, place, register_part
+from .linear import LINEAR_LIBRARIES, linear
+
+
+@register_part("mixer", "paged_attention")
+class PagedAttention(Part):
+    """Grouped-query attention: q/k/v projections without bias, a position
+    encoding on q and k, the new keys and values written into cache pages, then
+    every token attends its sequence's keys in the pages up to its own
+    position, and the output projection (lite_llama/models/llama.py:26-62 for a
+    prompt, :64-105 for one decoded token; here both are one path because the
+    kernels read only the cache). scale defaults to head_dim^-0.5 (llama.py:173).
+
+    The three projection matrices are concatenated at load into one
+    [(Hq + 2 Hkv) D, hidden] matrix, rows q | k | v (the reference fuses k and
+    v, lite_llama/executor/weight_convert.py:229-246)."""
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: Optional[Part] = None, scale: Optional[float] = None,
+                 window: Optional[int] = None,
+                 q_name: str = "q_proj.weight", k_name: str = "k_proj.weight",
+                 v_name: str = "v_proj.weight", o_name: str = "o_proj.weight"):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if head_dim % 2 or head_dim > 256:
+            raise ValueError(f"the attention kernels take even head sizes up to 256, got {head_dim}")
+        self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
+        self.num_kv_heads, self.head_dim = int(num_kv_heads), int(head_dim)
+        self.position = position
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.window = int(window) if window else None
+        self.names = (q_name, k_name, v_name, o_name)
+        self.q_size = self.num_heads * self.head_dim
+        self.kv_size = self.num_kv_heads * self.head_dim
+        self.qkv: Optional[torch.Tensor] = None
+        self.o: Optional[torch.Tensor] = None
+        libs = ("attention", "rope") + LINEAR_LIBRARIES
+        if position is not None:
+            libs += tuple(position.kernel_libraries)
+        self.kernel_libraries = tuple(dict.fromkeys(libs))
+
+    def cache_spec(self):
+        return PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
+
+    def param_sources(self) -> List[ParamSource]:
+        qn, kn, vn, on = self.names
+        return [ParamSource(qn, (self.q_size, self.hidden_size)),
+                ParamSource(kn, (self.kv_size, self.hidden_size)),
+                ParamSource(vn, (self.kv_size, self.hidden_size)),
+                ParamSource(on, (self.hidden_size, self.q_size))]
+
+    def load(self, tensors, dtype, device) -> None:
+        qn, kn, vn, on = self.names
+        self.qkv = place(torch.cat([tensors[qn], tensors[kn], tensors[vn]], dim=0),
+                         "matrix", dtype, device)
+        self.o = place(tensors[on], "matrix", dtype, device)
+        if self.position is not None:
+            self.position.load({}, dtype, device)
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        T = x.shape[0]
+        Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
+        qkv = linear(x, self.qkv)
+        q = qkv[:, :self.q_size].view(T, Hq, D)
+        k = qkv[:, self.q_size:self.q_size + self.kv_size].view(T, Hkv, D)
+        v = qkv[:, self.q_size + self.kv_size:].view(T, Hkv, D)
+        inv_freq = None
+        if self.position is not None:
+            inv_freq = self.position.rotary_inv_freq()
+            if inv_freq is None:
+                self.position.apply(q, k, ctx.positions)
+        group = ctx.groups[cache.group]
+        ops.rope_store(q, k, v, ctx.positions, inv_freq,
+                       group.slots if cache.writable else None, cache.k, cache.v,
+                       cache.page_size)
+        out = torch.empty((T, Hq, D), dtype=x.dtype, device=x.device)
+        ops.attention_generic(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
+                              group.block_table, ctx.work_seq, ctx.work_qoff, self.scale,
+                              self.window or 0)
+        return linear(out.view(T, Hq * D), self.o)

@@ -1,0 +1,105 @@
+"""What every part of a layer looks like to the rest of the engine.
+
+A model is put together from parts that know their own sizes and constants and
+nothing about the model they are in: an embedding, blocks (each a norm, a
+mixer, a norm and a feed-forward in some arrangement), a final norm and a head.
+Parts are chosen by name from the registries below, layer by layer, so one
+model may use different mixers and feed-forwards in different layers, and a new
+part is added by registering a class: no file of the engine changes.
+
+Interfaces
+----------
+every part:
+    kernel_libraries        names of the HIP libraries it launches (built on demand)
+    param_sources()         checkpoint tensors it wants: ParamSource(name, shape, kind),
+                            names relative to the prefix the model gives the part
+    load(tensors, dtype, device)   take them (keyed by the same names); may fuse
+norm:            forward(x, residual) -> (y, new_residual)    residual may be None
+mixer:           cache_spec() -> PagedKVSpec | StateSpec | None
+                 forward(x, ctx, cache) -> y      x, y: [T, hidden]
+feed-forward:    forward(x) -> y
+position:        rotary_inv_freq() -> float32 [D/2] or None;  apply(q, k, positions) in place
+embedding:       forward(token_ids int32 [T]) -> [T, hidden]
+head:            forward(x [R, hidden]) -> float32 logits [R, vocab]
+block:           forward(h, residual, ctx, cache) -> (h, residual)
+
+``ctx`` is the StepContext of engine/batch.py: the flat batch (positions,
+q_start, ctx_len, per cache group its block table and slot mapping, the state
+slot of every sequence). ``cache`` is the view of the one cache layer the call
+was given: for a paged spec .k/.v pools of that layer, .group, .writable; for a
+state spec .state [max_num_seqs, *shape].
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Dict, List, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSource:
+    name: str                 # relative to the part's prefix, e.g. "q_proj.weight"
+    shape: Tuple[int, ...]
+    kind: str = "matrix"      # "matrix": held in the engine dtype; "vector": held in float32;
+                              # "table": integers, held as int32
+
+
+@dataclass(frozen=True)
+class PagedKVSpec:
+    """Keys and values of every token, in pages; ``window``: only the last
+    ``window`` positions are ever read again, older pages can be given back."""
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """A tensor of fixed size per request (in the slot of the request)."""
+    shape: Tuple[int, ...]
+    dtype: Optional[torch.dtype] = None     # None: the engine dtype
+
+
+class Part:
+    kernel_libraries: Tuple[str, ...] = ()
+
+    def param_sources(self) -> List[ParamSource]:
+        return []
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device) -> None:
+        pass
+
+
+PART_KINDS = ("embedding", "norm", "mixer", "feed_forward", "position", "head", "block")
+PART_REGISTRY: Dict[str, Dict[str, Any]] = {k: {} for k in PART_KINDS}
+
+
+def register_part(kind: str, name: str):
+    """Class decorator: make ``name`` available for ``kind`` in layer specs."""
+    if kind not in PART_REGISTRY:
+        raise KeyError(f"unknown part kind {kind!r}; kinds: {PART_KINDS}")
+
+    def deco(cls):
+        PART_REGISTRY[kind][name] = cls
+        return cls
+    return deco
+
+
+def build_part(kind: str, name: str, **kwargs):
+    try:
+        cls = PART_REGISTRY[kind][name]
+    except KeyError:
+        raise KeyError(f"no {kind} part named {name!r}; registered: "
+                       f"{sorted(PART_REGISTRY.get(kind, {}))}") from None
+    return cls(**kwargs)
+
+
+def place(t: torch.Tensor, kind: str, dtype: torch.dtype, device) -> torch.Tensor:
+    """A checkpoint tensor as the engine holds it: matrices in the engine dtype,
+    vectors in float32, integer tables as int32."""
+    if kind == "vector":
+        return t.to(device=device, dtype=torch.float32).contiguous()
+    if kind == "table":
+        return t.to(device=device, dtype=torch.int32).contiguous()
+    return t.to(device=device, dtype=dtype).contiguous()

@@ -1,0 +1,41 @@
+"""The dense gated feed-forward."""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from .base import ParamSource, Part, place, register_part
+from .linear import LINEAR_LIBRARIES, linear
+
+
+@register_part("feed_forward", "swiglu")
+class SwiGLU(Part):
+    """down(silu(gate(x)) * up(x)), three matrices without bias
+    (lite_llama/models/llama.py:107-120, lite_llama/kernels/swiglu.py:44-67).
+    gate and up are concatenated at load into one [2I, hidden] matrix (rows
+    gate | up) so that one product feeds the SiLU-multiply kernel."""
+    kernel_libraries = ("activation",) + LINEAR_LIBRARIES
+
+    def __init__(self, hidden_size: int, intermediate_size: int,
+                 gate_name: str = "gate_proj.weight", up_name: str = "up_proj.weight",
+                 down_name: str = "down_proj.weight"):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.names = (gate_name, up_name, down_name)
+        self.gate_up: Optional[torch.Tensor] = None
+        self.down: Optional[torch.Tensor] = None
+
+    def param_sources(self) -> List[ParamSource]:
+        g, u, d = self.names
+        return [ParamSource(g, (self.intermediate_size, self.hidden_size)),
+                ParamSource(u, (self.intermediate_size, self.hidden_size)),
+                ParamSource(d, (self.hidden_size, self.intermediate_size))]
+
+    def load(self, tensors, dtype, device) -> None:
+        g, u, d = self.names
+        self.gate_up = place(torch.cat([tensors[g], tensors[u]], dim=0), "matrix", dtype, device)
+        self.down = place(tensors[d], "matrix", dtype, device)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return linear(ops.silu_mul(linear(x, self.gate_up)), self.down)

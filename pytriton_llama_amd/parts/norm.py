@@ -1,0 +1,34 @@
+"""RMSNorm with the residual sum fused in front of it."""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from .base import ParamSource, Part, place, register_part
+
+
+@register_part("norm", "rmsnorm")
+class RMSNorm(Part):
+    """y = (x + residual) * rsqrt(mean((x + residual)^2) + eps) * weight, with the
+    sum returned as the new residual (lite_llama/kernels/skip_rmsnorm.py:94-181;
+    call sites lite_llama/models/llama.py:149,160,219). Without a residual the
+    input itself is the residual (:181)."""
+    kernel_libraries = ("norm",)
+
+    def __init__(self, size: int, eps: float, weight_name: str = "weight"):
+        self.size = int(size)
+        self.eps = float(eps)
+        self.weight_name = weight_name
+        self.weight: Optional[torch.Tensor] = None
+
+    def param_sources(self) -> List[ParamSource]:
+        return [ParamSource(self.weight_name, (self.size,), "vector")]
+
+    def load(self, tensors, dtype, device) -> None:
+        self.weight = place(tensors[self.weight_name], "vector", dtype, device)
+
+    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor]):
+        y = ops.add_rmsnorm(x, residual, self.weight, self.eps)
+        return y, (x if residual is None else residual)

@@ -1,0 +1,80 @@
+"""Helpers of the GPU tests: model folders, the plain logits, in-process replay."""
+import os
+
+import torch
+
+import plain_llama
+from tiny_configs import tiny
+
+
+def make_folder(tmp_path_factory, name, seed=0, store_dtype=torch.float32, std=None):
+    from pytriton_llama_amd.weights import write_random_model
+    cfg, cstd, norm_std, page = tiny(name)
+    folder = str(tmp_path_factory.mktemp(f"tiny_{name}"))
+    write_random_model(cfg, folder, seed=seed, dtype=store_dtype, norm_std=norm_std,
+                       std=cstd if std is None else std)
+    return folder, page
+
+
+def random_sequences(vocab, lengths, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return {f"r{i}": torch.randint(0, vocab, (n,), generator=g).tolist()
+            for i, n in enumerate(lengths)}
+
+
+def plain_logits(folder, seqs, weights_as=torch.float32):
+    """Logits of the plain implementation, in float32 arithmetic, with weights
+    rounded to ``weights_as`` first (the values a bfloat16 engine holds)."""
+    cfg, w = plain_llama.read_model_folder(folder)
+    if weights_as != torch.float32:
+        w = {k: (v.to(weights_as).float() if v.dim() == 2 else v) for k, v in w.items()}
+    return {rid: plain_llama.forward(cfg, w, toks) for rid, toks in seqs.items()}
+
+
+def load_runner(folder, dtype, page_size, num_pages, device="cuda:0", max_num_seqs=8):
+    import pytriton_llama_amd  # noqa: F401
+    from pytriton_llama_amd.config import build_model, read_config_json
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_weights
+    model = build_model(read_config_json(folder))
+    load_weights(model, folder, dtype, device)
+    return ModelRunner(model, page_size, num_pages, max_num_seqs)
+
+
+def replay(runner, steps, seqs):
+    """Run trace steps in-process; returns {request: float32 [len, vocab]} on the CPU."""
+    from pytriton_llama_amd.engine.batch import StepEntry
+    V = runner.model.vocab_size
+    out = {rid: torch.full((len(t), V), float("nan")) for rid, t in seqs.items()}
+    fed = {rid: 0 for rid in seqs}
+    for st in steps:
+        entries = [StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]]
+        logits = runner.step(entries).float().cpu()
+        row = 0
+        for e in st["entries"]:
+            for w in e["want"]:
+                out[e["id"]][fed[e["id"]] + w] = logits[row]
+                row += 1
+            fed[e["id"]] += len(e["tokens"])
+        assert row == logits.shape[0]
+        for rid in st["end"]:
+            runner.end(rid)
+        runner.manager.check()
+    return out
+
+
+def first_mismatch(got, want, tol):
+    """(request, position, error) of the first place whose logits differ by more
+    than tol * (largest |logit| of the plain result), or None."""
+    for rid in want:
+        scale = float(want[rid].abs().max())
+        err = (got[rid] - want[rid]).abs().amax(dim=-1) / scale
+        err = torch.where(torch.isnan(err), torch.full_like(err, float("inf")), err)
+        bad = torch.nonzero(err > tol)
+        if len(bad):
+            p = int(bad[0])
+            return rid, p, float(err[p])
+    return None
+
+
+TOL = {torch.float32: 2e-4, torch.bfloat16: 4e-2}

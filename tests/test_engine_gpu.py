@@ -1,0 +1,102 @@
+"""The engine against the plain implementation under every way of cutting the
+work, in float32 and in bfloat16, for three tiny configurations."""
+import pytest
+import torch
+
+import cuttings
+from engine_helpers import (TOL, first_mismatch, load_runner, make_folder, plain_logits,
+                            random_sequences, replay)
+from tiny_configs import tiny
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [5, 9, 13, 17, 70, 41], "B": [31, 70, 100, 45, 64, 129], "C": [33, 80, 16, 97, 50]}
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def cases(tmp_path_factory, gpu_device):
+    out = {}
+    for name in ("A", "B", "C"):
+        folder, page = make_folder(tmp_path_factory, name, seed=11)
+        cfg = tiny(name)[0]
+        seqs = random_sequences(cfg["vocab_size"], LENGTHS[name], seed=5)
+        want = {torch.float32: plain_logits(folder, seqs),
+                torch.bfloat16: plain_logits(folder, seqs, torch.bfloat16)}
+        out[name] = (folder, page, seqs, want)
+    return out
+
+
+def run_cutting(cases, name, dtype, steps, num_pages=None):
+    folder, page, seqs, want = cases[name]
+    if num_pages is None:
+        num_pages = -(-cuttings.max_live_tokens(steps) // page)
+    runner = load_runner(folder, dtype, page, num_pages)
+    got = replay(runner, steps, seqs)
+    bad = first_mismatch(got, want[dtype], TOL[dtype])
+    assert bad is None, f"config {name} {dtype}: first wrong place (request, position, error) = {bad}"
+    assert all(g.pool.num_free == g.pool.num_pages for g in runner.manager.paged)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole(cases, name, dtype):
+    run_cutting(cases, name, dtype, cuttings.whole(cases[name][2]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_tokens_one_by_one(cases, name, dtype):
+    run_cutting(cases, name, dtype, cuttings.tail_decode(cases[name][2], 32))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(cases, name, dtype):
+    run_cutting(cases, name, dtype, cuttings.portions(cases[name][2]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_with_page_reuse(cases, name, dtype):
+    seqs = cases[name][2]
+    steps = cuttings.mixed(seqs, seed=3, max_live=4)
+    page = cases[name][1]
+    need = -(-cuttings.max_live_tokens(steps) // page)
+    total = sum(-(-len(t) // page) for t in seqs.values())
+    assert need < total, "the pool must be too small to hold all requests at once"
+    run_cutting(cases, name, dtype, steps, need)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_first_tokens_of_a_sequence(cases, dtype):
+    """Positions 0, 1, 2: one token whole, then one by one from an empty cache."""
+    folder, page, seqs, want = cases["B"]
+    toks = seqs["r0"][:3]
+    runner = load_runner(folder, dtype, page, 4)
+    from pytriton_llama_amd.engine.batch import StepEntry
+    got = []
+    for i, t in enumerate(toks):
+        got.append(runner.step([StepEntry("x", [t], [0])]).float().cpu()[0])
+    runner.end("x")
+    ref = want[dtype]["r0"][:3]
+    scale = float(ref.abs().max())
+    err = (torch.stack(got) - ref).abs().max() / scale
+    assert err < TOL[dtype], err
+    # the very first token attends only itself
+    one = runner.step([StepEntry("y", toks[:1], [0])]).float().cpu()[0]
+    assert (one - ref[0]).abs().max() / scale < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_long_decoding(cases, dtype):
+    """A short prompt and then 300 tokens one by one across many pages."""
+    folder, page, _, _ = cases["A"]
+    cfg = tiny("A")[0]
+    seqs = random_sequences(cfg["vocab_size"], [308], seed=9)
+    want = plain_logits(folder, seqs, dtype)
+    steps = cuttings.tail_decode(seqs, tail=300)
+    runner = load_runner(folder, dtype, page, -(-320 // page))
+    got = replay(runner, steps, seqs)
+    bad = first_mismatch(got, want, TOL[dtype])
+    assert bad is None, bad

@@ -1,0 +1,283 @@
+"""Each HIP kernel alone against a plain float32 torch formula of the same
+operation, at sizes other than the engine tests use."""
+import math
+
+import pytest
+import torch
+
+import plain_llama
+
+pytestmark = pytest.mark.gpu
+
+DT = [torch.float32, torch.bfloat16]
+IDS = ["fp32", "bf16"]
+
+
+def tol(dtype):
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+@pytest.fixture(scope="module")
+def ops(gpu_device):
+    from pytriton_llama_amd import ops
+    return ops
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+def test_embedding(ops, dtype):
+    table = torch.randn(301, 72, device="cuda").to(dtype)
+    ids = torch.tensor([0, 300, 5, 5, 17], dtype=torch.int32, device="cuda")
+    assert torch.equal(ops.embedding(table, ids), table[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+@pytest.mark.parametrize("shape", [(5, 72), (3, 2048), (2, 5000), (1, 16)])
+def test_add_rmsnorm(ops, dtype, shape):
+    torch.manual_seed(0)
+    x = torch.randn(shape, device="cuda").to(dtype)
+    r = torch.randn(shape, device="cuda").to(dtype)
+    w = (1 + 0.1 * torch.randn(shape[1], device="cuda")).float()
+    eps = 1e-3
+    want_y, want_r = plain_llama.add_rms_norm(x.float().cpu(), r.float().cpu(), w.cpu(), eps)
+    res = r.clone()
+    y = ops.add_rmsnorm(x, res, w, eps)
+    torch.testing.assert_close(y.float().cpu(), want_y, **tol(dtype))
+    torch.testing.assert_close(res.float().cpu(), want_r.to(dtype).float(), atol=0, rtol=0)
+    # without a residual: the input stays what it is
+    x2 = x.clone()
+    y2 = ops.add_rmsnorm(x2, None, w, eps)
+    torch.testing.assert_close(y2.float().cpu(), plain_llama.rms_norm(x.float().cpu(), w.cpu(), eps),
+                               **tol(dtype))
+    assert torch.equal(x2, x)
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+def test_silu_mul(ops, dtype):
+    torch.manual_seed(1)
+    gu = (3 * torch.randn(7, 2 * 200, device="cuda")).to(dtype)
+    want = plain_llama.silu(gu[:, :200].float()) * gu[:, 200:].float()
+    torch.testing.assert_close(ops.silu_mul(gu).float(), want, **tol(dtype))
+    z = torch.zeros(1, 8, device="cuda", dtype=dtype)
+    assert torch.all(ops.silu_mul(z) == 0)
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+@pytest.mark.parametrize("mnk", [(1, 300, 72), (7, 65, 130), (130, 257, 96), (64, 64, 16), (3, 1000, 2050)])
+def test_gemm_nt(ops, dtype, mnk):
+    M, N, K = mnk
+    torch.manual_seed(2)
+    x = torch.randn(M, K, device="cuda").to(dtype)
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(dtype)
+    want = (x.double() @ w.double().T).float()
+    y = ops.gemm_nt(x, w)
+    torch.testing.assert_close(y.float(), want, **tol(dtype))
+    if dtype == torch.bfloat16:
+        y32 = ops.gemm_nt(x, w, torch.float32)
+        torch.testing.assert_close(y32, want, atol=1e-4, rtol=1e-4)
+    # strided rows of x (a slice of a wider buffer)
+    wide = torch.randn(M, K + 24, device="cuda").to(dtype)
+    ys = ops.gemm_nt(wide[:, 8:8 + K], w)
+    torch.testing.assert_close(ys.float(), (wide[:, 8:8 + K].double() @ w.double().T).float(),
+                               **tol(dtype))
+
+
+def _rope_reference(x, positions, inv_freq):
+    cos, sin = plain_llama.rope_cos_sin(inv_freq, positions)
+    return plain_llama.apply_rope(x, cos, sin)
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+@pytest.mark.parametrize("dims", [(5, 2, 48, 4), (3, 1, 128, 16), (4, 4, 8, 2)])
+def test_rope_store(ops, dtype, dims):
+    Hq, Hkv, D, P = dims
+    T = 9
+    torch.manual_seed(3)
+    width = (Hq + 2 * Hkv) * D
+    qkv = torch.randn(T, width, device="cuda").to(dtype)
+    orig = qkv.clone()
+    q = qkv[:, :Hq * D].view(T, Hq, D)
+    k = qkv[:, Hq * D:(Hq + Hkv) * D].view(T, Hkv, D)
+    v = qkv[:, (Hq + Hkv) * D:].view(T, Hkv, D)
+    positions = torch.tensor([0, 1, 2, 77, 1000, 4095, 8191, 100000, 5], dtype=torch.int32, device="cuda")
+    inv_freq = plain_llama.rope_inv_freq_default(500000.0, D)
+    pages = 7
+    kc = torch.zeros(pages, Hkv, P, D, device="cuda", dtype=dtype)
+    vc = torch.zeros_like(kc)
+    slots = torch.randperm(pages * P)[:T].to(torch.int32).cuda()
+    ops.rope_store(q, k, v, positions, inv_freq.cuda(), slots, kc, vc, P)
+    o = orig.float().cpu()
+    want_q = _rope_reference(o[:, :Hq * D].view(T, Hq, D), positions.cpu(), inv_freq)
+    want_k = _rope_reference(o[:, Hq * D:(Hq + Hkv) * D].view(T, Hkv, D), positions.cpu(), inv_freq)
+    torch.testing.assert_close(q.float().cpu(), want_q, **tol(dtype))
+    # k in the projection buffer is untouched, the cache holds the rotated k and v
+    assert torch.equal(k, orig[:, Hq * D:(Hq + Hkv) * D].view(T, Hkv, D))
+    for t in range(T):
+        page, off = int(slots[t]) // P, int(slots[t]) % P
+        torch.testing.assert_close(kc[page, :, off].float().cpu(), want_k[t], **tol(dtype))
+        assert torch.equal(vc[page, :, off], v[t])
+    # untouched slots stay zero
+    mask = torch.ones(pages * P, dtype=torch.bool)
+    mask[slots.long().cpu()] = False
+    assert torch.all(kc.permute(0, 2, 1, 3).reshape(pages * P, -1)[mask.cuda()] == 0)
+
+
+def _paged_setup(seq_lens, q_lens, Hkv, D, P, dtype, seed, shuffle=True):
+    """Random keys/values laid into shuffled pages; returns tensors and the dense copies."""
+    g = torch.Generator().manual_seed(seed)
+    n = len(seq_lens)
+    pages_per = [-(-s // P) for s in seq_lens]
+    total = sum(pages_per) + 3
+    perm = torch.randperm(total, generator=g).tolist() if shuffle else list(range(total))
+    kc = torch.randn(total, Hkv, P, D, generator=g).to(dtype)    # garbage everywhere first
+    vc = torch.randn(total, Hkv, P, D, generator=g).to(dtype)
+    maxp = max(pages_per)
+    bt = torch.full((n, maxp), -1, dtype=torch.int32)
+    dense_k, dense_v = [], []
+    it = iter(perm)
+    for i, s in enumerate(seq_lens):
+        k = torch.randn(s, Hkv, D, generator=g).to(dtype)
+        v = torch.randn(s, Hkv, D, generator=g).to(dtype)
+        dense_k.append(k.float())
+        dense_v.append(v.float())
+        for j in range(pages_per[i]):
+            pg = next(it)
+            bt[i, j] = pg
+            lo, hi = j * P, min(s, (j + 1) * P)
+            kc[pg, :, :hi - lo] = k[lo:hi].transpose(0, 1)
+            vc[pg, :, :hi - lo] = v[lo:hi].transpose(0, 1)
+    return kc, vc, bt, dense_k, dense_v
+
+
+def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=0, boost=None):
+    kc, vc, bt, dk, dv = _paged_setup(seq_lens, q_lens, Hkv, D, P, dtype, seed)
+    g = torch.Generator().manual_seed(seed + 100)
+    T = sum(q_lens)
+    q = torch.randn(T, Hq, D, generator=g).to(dtype)
+    if boost is not None:
+        boost(q, dk, kc, bt)
+    q_start = [0]
+    for ql in q_lens:
+        q_start.append(q_start[-1] + ql)
+    work_seq, work_qoff = [], []
+    for s, ql in enumerate(q_lens):
+        for off in range(0, ql, 16):
+            work_seq.append(s)
+            work_qoff.append(off)
+    dev = "cuda"
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    out = torch.zeros(T, Hq, D, dtype=dtype, device=dev)
+    scale = 1.0 / math.sqrt(D)
+    ops.attention_generic(out, q.to(dev), kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
+                          bt.to(dev), i32(work_seq), i32(work_qoff), scale, window)
+    # plain: full causal attention over the sequence, rows of the portion kept
+    for i, (s, ql) in enumerate(zip(seq_lens, q_lens)):
+        full_q = torch.zeros(s, Hq, D)
+        full_q[s - ql:] = q[q_start[i]:q_start[i + 1]].float()
+        want = plain_llama.causal_attention(full_q, dk[i], dv[i], scale,
+                                            window if window else None)[s - ql:]
+        got = out[q_start[i]:q_start[i + 1]].float().cpu()
+        torch.testing.assert_close(got, want, **tol(dtype), msg=lambda m: f"sequence {i}: {m}")
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+@pytest.mark.parametrize("case", [
+    dict(seq_lens=[40], q_lens=[40], Hq=4, Hkv=4, D=64, P=16),            # whole prompt, MHA
+    dict(seq_lens=[37, 5, 130], q_lens=[1, 1, 1], Hq=8, Hkv=2, D=48, P=4),  # decode, GQA
+    dict(seq_lens=[100, 64, 33], q_lens=[30, 1, 33], Hq=6, Hkv=1, D=128, P=8),  # mixed, MQA
+    dict(seq_lens=[70], q_lens=[19], Hq=2, Hkv=1, D=256, P=5),            # big heads, odd page size
+    dict(seq_lens=[50, 21], q_lens=[17, 2], Hq=4, Hkv=2, D=8, P=3),       # tiny heads
+])
+def test_attention_generic(ops, dtype, case):
+    _attention_case(ops, dtype, **case)
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+def test_attention_window(ops, dtype):
+    _attention_case(ops, dtype, seq_lens=[90, 40], q_lens=[25, 1], Hq=4, Hkv=2, D=32, P=8, window=20)
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+def test_attention_far_key_stands_out(ops, dtype):
+    """One early key is made to dominate the last query's scores, so a kernel
+    that drops or misplaces a far page fails."""
+    def boost(q, dk, kc, bt):
+        # key 3 of sequence 0 (first page) aligned with the last query, head 0
+        direction = torch.ones(32) * 3.0
+        q[-1, :, :] = direction.to(q.dtype)
+        page = int(bt[0, 0])
+        kc[page, :, 3] = direction.to(kc.dtype)
+        dk[0][3] = direction
+    _attention_case(ops, dtype, seq_lens=[300], q_lens=[1], Hq=2, Hkv=1, D=32, P=16, boost=boost)
+
+
+def test_attention_page_placement_does_not_matter(ops):
+    """The same keys in differently permuted pages give the same output bit for bit."""
+    outs = []
+    for shuffle_seed in (0, 1):
+        kc, vc, bt, dk, dv = _paged_setup([75], [75], 2, 32, 8, torch.float32, seed=4, shuffle=True)
+        if shuffle_seed:
+            perm = torch.randperm(kc.shape[0], generator=torch.Generator().manual_seed(99))
+            inv = torch.empty_like(perm)
+            inv[perm] = torch.arange(len(perm))
+            kc, vc = kc[perm], vc[perm]
+            bt = torch.where(bt >= 0, inv[bt.clamp(min=0).long()].to(torch.int32), bt)
+        q = torch.randn(75, 4, 32, generator=torch.Generator().manual_seed(8))
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+        out = torch.zeros(75, 4, 32, device="cuda")
+        ops.attention_generic(out, q.cuda(), kc.cuda(), vc.cuda(), i32([0, 75]), i32([75]),
+                              bt.cuda(), i32([0, 0, 0, 0, 0]), i32([0, 16, 32, 48, 64]),
+                              1 / math.sqrt(32), 0)
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[1])
+
+
+def test_argmax(ops):
+    torch.manual_seed(5)
+    logits = torch.randn(6, 1003, device="cuda")
+    logits[2, 7] = logits[2, 900] = 50.0       # a tie goes to the lowest id
+    got = ops.argmax(logits).cpu()
+    want = torch.argmax(logits.cpu(), dim=-1)
+    want[2] = 7
+    assert got.tolist() == want.tolist()
+
+
+def test_sample_top_p_distribution(ops):
+    """The kernel's nucleus equals the plain rule's, and the draw follows it."""
+    torch.manual_seed(6)
+    R, V = 5, 777
+    logits = (3 * torch.randn(R, V)).cuda()
+    temperature = torch.tensor([0.8, 1.0, 0.5, 2.0, 0.7]).cuda()
+    top_p = torch.tensor([0.9, 1.0, 0.3, 0.95, 1e-6]).cuda()
+    u = torch.tensor([0.0, 0.5, 0.999, 0.25, 0.7]).cuda()
+    tok, probs = ops.sample_top_p(logits, temperature, top_p, u, return_probs=True)
+    for r in range(R):
+        want = plain_llama.top_p_probs(logits[r].cpu(), float(temperature[r]), float(top_p[r]))
+        torch.testing.assert_close(probs[r].cpu().double(), want, atol=1e-5, rtol=1e-4)
+        # inverse CDF in vocabulary order
+        cdf = torch.cumsum(want, 0)
+        expect = int(torch.searchsorted(cdf, torch.tensor(float(u[r]), dtype=torch.double), right=True))
+        got = int(tok[r])
+        assert want[got] > 0
+        assert abs(float(cdf[got]) - float(cdf[min(expect, V - 1)])) < 1e-4 or got == expect
+    # top_p -> 0 is greedy
+    assert int(tok[4]) == int(torch.argmax(logits[4]))
+
+
+def test_sample_top_p_frequencies(ops):
+    """Many draws with different uniforms reproduce the probabilities."""
+    logits = torch.tensor([[2.0, 1.0, 0.0, -1.0, 0.5, -30.0]]).cuda().repeat(4000, 1)
+    t = torch.full((4000,), 1.0).cuda()
+    p = torch.full((4000,), 0.9).cuda()
+    u = torch.rand(4000, generator=torch.Generator().manual_seed(1)).cuda()
+    tok = ops.sample_top_p(logits, t, p, u).cpu()
+    want = plain_llama.top_p_probs(logits[0].cpu(), 1.0, 0.9)
+    freq = torch.bincount(tok.long(), minlength=6).double() / 4000
+    assert torch.all((freq - want).abs() < 0.03), (freq, want)
+    assert freq[want == 0].sum() == 0
+
+
+def test_kernels_refuse_cpu_tensors(ops):
+    with pytest.raises(ops.KernelError):
+        ops.silu_mul(torch.zeros(2, 4))
+    with pytest.raises(ops.KernelError):
+        ops.add_rmsnorm(torch.zeros(2, 20000, device="cuda"), None, torch.ones(20000, device="cuda"), 1e-5)
