@@ -123,7 +123,8 @@ def rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: tor
         raise KernelError("rope_store: k and v must be [T, Hkv, D]")
     rs = q.stride(0)
     for name, t in (("q", q), ("k", k), ("v", v)):
-        if t.stride(2) != 1 or t.stride(1) != D or t.stride(0) != rs or t.dtype != q.dtype:
+        if t.stride(2) != 1 or (t.shape[1] > 1 and t.stride(1) != D) or (T > 1 and t.stride(0) != rs) \
+                or t.dtype != q.dtype:
             raise KernelError(f"rope_store: {name} must be a [T, heads, D] view with dense heads "
                               "and the common row stride")
     _i32(positions, "positions")
@@ -192,7 +193,7 @@ def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         raise KernelError(f"attention: head size {D} exceeds the kernel's limit of 256")
     if Hq % Hkv:
         raise KernelError(f"attention: {Hq} query heads are not a multiple of {Hkv} kv heads")
-    if q.stride(2) != 1 or q.stride(1) != D or out.stride(2) != 1 or out.stride(1) != D:
+    if q.stride(2) != 1 or out.stride(2) != 1 or (Hq > 1 and (q.stride(1) != D or out.stride(1) != D)):
         raise KernelError("attention: q and out need dense heads")
     if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
         raise KernelError("attention: q, out and the caches must share one dtype")

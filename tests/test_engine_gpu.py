@@ -62,7 +62,7 @@ def test_mixed_with_page_reuse(cases, name, dtype):
     seqs = cases[name][2]
     steps = cuttings.mixed(seqs, seed=3, max_live=4)
     page = cases[name][1]
-    need = -(-cuttings.max_live_tokens(steps) // page)
+    need = cuttings.max_live_tokens(steps, round_to=page) // page
     total = sum(-(-len(t) // page) for t in seqs.values())
     assert need < total, "the pool must be too small to hold all requests at once"
     run_cutting(cases, name, dtype, steps, need)
