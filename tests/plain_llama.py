@@ -184,7 +184,7 @@ def swiglu_mlp(x, w, prefix):
 # whole model
 # --------------------------------------------------------------------------
 def forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int],
-            return_hidden: bool = False) -> torch.Tensor:
+            return_hidden: bool = False, first_position: int = 0) -> torch.Tensor:
     """Logits [S, V] of one whole sequence. lite_llama/models/llama.py:189-223:
     embedding, then per layer (llama.py:149-162) add+norm, attention, add+norm,
     MLP with the residual carried beside the hidden state, a last add+norm
@@ -194,7 +194,7 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int],
     dtype = w["model.embed_tokens.weight"].dtype
     eps = float(cfg.get("rms_norm_eps", 1e-5))
     h = w["model.embed_tokens.weight"][ids]
-    cos, sin = rope_cos_sin(rope_inv_freq(cfg), torch.arange(len(ids)))
+    cos, sin = rope_cos_sin(rope_inv_freq(cfg), first_position + torch.arange(len(ids)))
     cos, sin = cos.to(dtype), sin.to(dtype)
     residual = None
     for i in range(cfg["num_hidden_layers"]):

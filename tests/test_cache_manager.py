@@ -1,0 +1,143 @@
+"""The cache manager on the CPU: no page lost, held twice or freed twice,
+under random orders of requests; windows give pages back; slots."""
+import random
+
+import pytest
+
+from pytriton_llama_amd.cache import RELEASED, CacheManager, OutOfPages, OutOfSlots, PagePool
+from pytriton_llama_amd.parts import PagedKVSpec, StateSpec
+
+FULL = PagedKVSpec(2, 16)
+WIN = PagedKVSpec(2, 16, window=10)
+
+
+def test_nine_pages_like_the_reference_scenarios():
+    """The 9-block scenarios of the reference's tests/test_mem_manager.py:26-183
+    (alloc 3; alloc 10 fails and leaves the state; release then alloc again;
+    free everything), on pages."""
+    m = CacheManager([FULL], page_size=1, num_pages=9, max_num_seqs=4)
+    m.admit("a")
+    m.append("a", 3)
+    assert m.paged[0].pool.num_free == 6 and len(m.block_table("a", 0)) == 3
+    m.admit("b")
+    assert not m.can_append("b", 10)
+    with pytest.raises(OutOfPages):
+        m.append("b", 10)
+    assert m.paged[0].pool.num_free == 6 and m.num_tokens["b"] == 0   # nothing was taken
+    m.append("b", 4)
+    held = set(m.block_table("a", 0))
+    m.free("a")
+    assert m.paged[0].pool.num_free == 5
+    m.admit("c")
+    m.append("c", 3)
+    assert set(m.block_table("c", 0)) == held                           # freed pages are used again
+    m.free("b")
+    m.free("c")
+    assert m.paged[0].pool.num_free == 9
+    m.check()
+
+
+def test_pages_grow_with_tokens_and_slots_address_them():
+    m = CacheManager([FULL, FULL], page_size=4, num_pages=5, max_num_seqs=2)
+    assert len(m.paged) == 1 and m.paged[0].layers == [0, 1]        # same needs: one group
+    m.admit("a")
+    assert m.append("a", 5) == 0
+    assert m.pages_needed("a", 3) == [0] and m.pages_needed("a", 4) == [1]
+    assert m.append("a", 3) == 5
+    t = m.block_table("a", 0)
+    assert len(t) == 2
+    assert m.slots("a", 0, 3, 3) == [t[0] * 4 + 3, t[1] * 4 + 0, t[1] * 4 + 1]
+
+
+def test_double_free_and_unknown_requests_raise():
+    m = CacheManager([FULL], 4, 4, 2)
+    m.admit("a")
+    m.append("a", 4)
+    m.free("a")
+    with pytest.raises(RuntimeError):
+        m.free("a")
+    with pytest.raises(RuntimeError):
+        m.append("zz", 1)
+    pool = PagePool(3)
+    p = pool.take(2)
+    pool.give_back(p)
+    with pytest.raises(RuntimeError):
+        pool.give_back(p[:1])
+
+
+def test_state_slots():
+    m = CacheManager([FULL, StateSpec((3, 5)), None], 4, 4, max_num_seqs=2)
+    assert m.layer_home == [("paged", 0, 0), ("state", 0, 0), None]
+    s = {m.admit("a"), m.admit("b")}
+    assert s == {0, 1} and m.num_free_slots == 0
+    with pytest.raises(OutOfSlots):
+        m.admit("c")
+    with pytest.raises(RuntimeError):
+        m.admit("a")
+    sa = m.slot_of["a"]
+    m.free("a")
+    assert m.admit("c") == sa
+    m.check()
+
+
+def test_groups_with_different_needs_have_their_own_pages():
+    m = CacheManager([FULL, WIN, FULL, WIN], page_size=4, num_pages=[8, 4], max_num_seqs=2)
+    assert [g.layers for g in m.paged] == [[0, 2], [1, 3]]
+    m.admit("a")
+    m.append("a", 16)                       # 4 pages in both groups
+    assert [g.pool.num_free for g in m.paged] == [4, 0]
+    assert m.release_behind_window("a") == 1
+    # a query at position 16 reads keys 7..16: page 0 (keys 0-3) is dead, page 1 (4-7) still holds key 7
+    assert m.block_table("a", 1)[0] == RELEASED and m.block_table("a", 1)[1] >= 0
+    assert [g.pool.num_free for g in m.paged] == [4, 1]
+    assert m.can_append("a", 4) and not m.can_append("a", 5)
+    m.append("a", 4)
+    m.release_behind_window("a")
+    assert m.block_table("a", 1)[:2] == [RELEASED, RELEASED]
+    with pytest.raises(RuntimeError):
+        m.slots("a", 1, 0, 1)
+    m.check()
+    m.free("a")
+    assert [g.pool.num_free for g in m.paged] == [8, 4]
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_keep_the_books(seed):
+    rng = random.Random(seed)
+    m = CacheManager([FULL, WIN, StateSpec((2,))], page_size=rng.choice([1, 4, 16]),
+                     num_pages=[rng.randint(6, 30), rng.randint(6, 30)], max_num_seqs=5)
+    live, n = {}, 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and m.num_free_slots:
+            rid = f"r{n}"
+            n += 1
+            m.admit(rid)
+            live[rid] = 0
+        elif op < 0.8 and live:
+            rid = rng.choice(list(live))
+            k = rng.randint(1, 20)
+            before = [g.pool.num_free for g in m.paged]
+            if m.can_append(rid, k):
+                assert m.append(rid, k) == live[rid]
+                live[rid] += k
+                m.release_behind_window(rid)
+            else:
+                with pytest.raises(OutOfPages):
+                    m.append(rid, k)
+                assert [g.pool.num_free for g in m.paged] == before
+        elif live:
+            rid = rng.choice(list(live))
+            m.free(rid)
+            del live[rid]
+        m.check()
+        for rid, cnt in live.items():
+            assert m.num_tokens[rid] == cnt
+            full, win = m.block_table(rid, 0), m.block_table(rid, 1)
+            assert len(full) == -(-cnt // m.page_size) and all(p >= 0 for p in full)
+            first = max(0, cnt - 10 + 1) // m.page_size
+            assert all((p == RELEASED) == (i < first) for i, p in enumerate(win))
+    for rid in list(live):
+        m.free(rid)
+    m.check()
+    assert all(g.pool.num_free == g.pool.num_pages for g in m.paged) and m.num_free_slots == 5

@@ -1,0 +1,200 @@
+"""Each part alone on the GPU, and a model put together from the package's parts
+and the tests' toy parts: a mixer with state of its own beside windowed paged
+attention, another norm, another feed-forward, a layer that runs twice."""
+import copy
+import math
+
+import pytest
+import torch
+
+import cuttings
+import plain_llama
+import toy_parts  # noqa: F401
+from engine_helpers import replay
+
+pytestmark = pytest.mark.gpu
+
+
+def test_rmsnorm_part(gpu_device):
+    from pytriton_llama_amd.parts import build_part
+    n = build_part("norm", "rmsnorm", size=72, eps=1e-3)
+    w = 1 + 0.1 * torch.randn(72)
+    n.load({"weight": w}, torch.float32, gpu_device)
+    x, r = torch.randn(5, 72), torch.randn(5, 72)
+    y, res = n.forward(x.cuda(), r.clone().cuda())
+    wy, wr = plain_llama.add_rms_norm(x, r, w, 1e-3)
+    torch.testing.assert_close(y.cpu(), wy, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(res.cpu(), wr)
+    xc = x.cuda()
+    y0, res0 = n.forward(xc, None)
+    assert res0 is xc
+
+
+def test_rotary_part_alone(gpu_device):
+    from pytriton_llama_amd.parts import build_part
+    sc = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+              original_max_position_embeddings=64)
+    rot = build_part("position", "rotary", head_dim=32, theta=5e5, **sc)
+    torch.testing.assert_close(rot.inv_freq_host, plain_llama.rope_inv_freq_llama3(5e5, 32, sc))
+    rot.load({}, torch.float32, gpu_device)
+    buf = torch.randn(6, (3 + 1) * 32, device="cuda")
+    orig = buf.cpu().clone()
+    q, k = buf[:, :96].view(6, 3, 32), buf[:, 96:].view(6, 1, 32)
+    pos = torch.tensor([0, 1, 63, 64, 500, 9], dtype=torch.int32, device="cuda")
+    rot.apply(q, k, pos)
+    cos, sin = plain_llama.rope_cos_sin(rot.inv_freq_host, pos.cpu())
+    torch.testing.assert_close(q.cpu(), plain_llama.apply_rope(orig[:, :96].view(6, 3, 32), cos, sin),
+                               atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(k.cpu(), plain_llama.apply_rope(orig[:, 96:].view(6, 1, 32), cos, sin),
+                               atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_swiglu_part(gpu_device, dtype):
+    from pytriton_llama_amd.parts import build_part
+    ff = build_part("feed_forward", "swiglu", hidden_size=72, intermediate_size=200)
+    w = {"gate_proj.weight": 0.1 * torch.randn(200, 72), "up_proj.weight": 0.1 * torch.randn(200, 72),
+         "down_proj.weight": 0.1 * torch.randn(72, 200)}
+    ff.load(w, dtype, gpu_device)
+    x = torch.randn(9, 72)
+    wr = {k: v.to(dtype).float() for k, v in w.items()}
+    want = plain_llama.swiglu_mlp(x.to(dtype).float(), wr, "")
+    got = ff.forward(x.to(dtype).cuda()).float().cpu()
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    torch.testing.assert_close(got, want, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_embedding_and_head_parts(gpu_device, dtype):
+    from pytriton_llama_amd.parts import build_part
+    emb = build_part("embedding", "token_embedding", vocab_size=300, hidden_size=72)
+    table = torch.randn(300, 72)
+    emb.load({"weight": table}, dtype, gpu_device)
+    ids = torch.tensor([0, 299, 7], dtype=torch.int32, device="cuda")
+    x = emb.forward(ids)
+    assert torch.equal(x.cpu(), table.to(dtype)[[0, 299, 7]])
+    head = build_part("head", "linear_head", vocab_size=300, hidden_size=72, tied_to=emb)
+    assert head.param_sources() == []
+    logits = head.forward(x)
+    assert logits.dtype == torch.float32
+    want = table.to(dtype).float()[[0, 299, 7]] @ table.to(dtype).float().T
+    torch.testing.assert_close(logits.cpu(), want, atol=1e-4, rtol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_attention_part_alone(gpu_device, dtype):
+    """The mixer with a cache of its own, fed in two portions, against plain
+    attention over the whole sequence; scale and window are parameters."""
+    from pytriton_llama_amd.cache import CacheManager, CacheStorage
+    from pytriton_llama_amd.engine.batch import StepEntry, build_context
+    from pytriton_llama_amd.parts import build_part
+    H, Hq, Hkv, D, S = 40, 4, 2, 16, 37
+    for window, scale in ((None, None), (9, 0.5)):
+        pos = build_part("position", "rotary", head_dim=D, theta=100.0)
+        att = build_part("mixer", "paged_attention", hidden_size=H, num_heads=Hq, num_kv_heads=Hkv,
+                         head_dim=D, position=pos, scale=scale, window=window)
+        g = torch.Generator().manual_seed(3)
+        w = {n: 0.15 * torch.randn(s, generator=g) for n, s in
+             (("q_proj.weight", (Hq * D, H)), ("k_proj.weight", (Hkv * D, H)),
+              ("v_proj.weight", (Hkv * D, H)), ("o_proj.weight", (H, Hq * D)))}
+        att.load(w, dtype, gpu_device)
+        x = torch.randn(S, H, generator=g).to(dtype)
+        mgr = CacheManager([att.cache_spec()], 4, 12, 2)
+        store = CacheStorage(mgr, dtype, gpu_device)
+        mgr.admit("r")
+        ys = []
+        for lo, hi in ((0, 20), (20, 37)):
+            ctx, _ = build_context([StepEntry("r", [0] * (hi - lo), [])], mgr, gpu_device)
+            ys.append(att.forward(x[lo:hi].cuda(), ctx, store.view(0)))
+            mgr.release_behind_window("r")
+        got = torch.cat(ys).float().cpu()
+        wr = {k: v.to(dtype).float() for k, v in w.items()}
+        xf = x.float()
+        q = (xf @ wr["q_proj.weight"].T).view(S, Hq, D)
+        k = (xf @ wr["k_proj.weight"].T).view(S, Hkv, D)
+        v = (xf @ wr["v_proj.weight"].T).view(S, Hkv, D)
+        cos, sin = plain_llama.rope_cos_sin(plain_llama.rope_inv_freq_default(100.0, D), torch.arange(S))
+        o = plain_llama.causal_attention(plain_llama.apply_rope(q, cos, sin),
+                                         plain_llama.apply_rope(k, cos, sin), v,
+                                         scale or 1 / math.sqrt(D), window)
+        want = o.reshape(S, Hq * D) @ wr["o_proj.weight"].T
+        # error relative to the largest output, as for logits: 2e-4 in float32; in bfloat16
+        # q, k, v, the attention output and the result are each rounded to 8 bits
+        err = float((got - want).abs().max() / want.abs().max())
+        assert err < (2e-4 if dtype == torch.float32 else 3e-2), err
+        if window:
+            assert mgr.block_table("r", 0)[0] == -1          # pages behind the window went back
+
+
+HYBRID = {"architectures": ["ToyStateLM"], "vocab_size": 90, "hidden_size": 48, "inner": 100,
+          "layers": ["state", "attention", "attention"], "order": [0, 1, 2, 1], "decay": 0.7,
+          "toy_norm": False, "toy_ffn": False, "heads": 3, "kv_heads": 1, "head_dim": 16,
+          "window": 24, "initializer_range": 0.25}
+
+
+def hybrid_plain(model, ids):
+    """Whole-sequence forward of the hybrid toy model with plain formulas."""
+    dev = "cpu"
+    x = model.embedding.weight.float().cpu()[torch.as_tensor(ids)]
+    h, residual = x, None
+    for call in model.schedule:
+        b = model.blocks[call.block]
+        h, residual = plain_llama.add_rms_norm(h, residual, b.input_norm.weight.cpu(), b.input_norm.eps)
+        m = b.mixer
+        if hasattr(m, "decay"):
+            u = h @ m.w.float().cpu().T
+            s = torch.zeros(u.shape[1])
+            ys = []
+            for t in range(u.shape[0]):
+                s = m.decay * s + u[t]
+                ys.append(s)
+            h = torch.stack(ys)
+        else:
+            S = h.shape[0]
+            qkv = h @ m.qkv.float().cpu().T
+            q = qkv[:, :m.q_size].view(S, m.num_heads, m.head_dim)
+            k = qkv[:, m.q_size:m.q_size + m.kv_size].view(S, m.num_kv_heads, m.head_dim)
+            v = qkv[:, m.q_size + m.kv_size:].view(S, m.num_kv_heads, m.head_dim)
+            cos, sin = plain_llama.rope_cos_sin(m.position.inv_freq_host, torch.arange(S))
+            o = plain_llama.causal_attention(plain_llama.apply_rope(q, cos, sin),
+                                             plain_llama.apply_rope(k, cos, sin), v, m.scale, m.window)
+            h = o.reshape(S, -1) @ m.o.float().cpu().T
+        h, residual = plain_llama.add_rms_norm(h, residual, b.post_norm.weight.cpu(), b.post_norm.eps)
+        ff = b.feed_forward
+        gu = h @ ff.gate_up.float().cpu().T
+        I = ff.intermediate_size
+        h = (plain_llama.silu(gu[:, :I]) * gu[:, I:]) @ ff.down.float().cpu().T
+    h, _ = plain_llama.add_rms_norm(h, residual, model.final_norm.weight.cpu(), model.final_norm.eps)
+    return h @ model.head.weight.float().cpu().T
+
+
+def test_toy_state_mixer_beside_windowed_attention(gpu_device):
+    """Registered, built and stepped without a change to the package: layer 0
+    keeps a state vector per request, layers 1 and 2 keep windowed keys in pages
+    (given back as the window moves on), and layer 1 runs twice with a memory for
+    each run. All cuttings agree with the plain whole-sequence result."""
+    from pytriton_llama_amd.config import build_model
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_random_weights
+    model = build_model(copy.deepcopy(HYBRID))
+    load_random_weights(model, 9, torch.float32, gpu_device, norm_std=0.1)
+    g = torch.Generator().manual_seed(6)
+    seqs = {f"r{i}": torch.randint(0, 90, (n,), generator=g).tolist()
+            for i, n in enumerate([70, 35, 101, 64, 50])}
+    want = {rid: hybrid_plain(model, t) for rid, t in seqs.items()}
+    for steps in (cuttings.whole(seqs), cuttings.tail_decode(seqs, 32), cuttings.portions(seqs),
+                  cuttings.mixed(seqs, seed=2)):
+        runner = ModelRunner(model, page_size=8, num_pages=40, max_num_seqs=4)
+        assert len(runner.manager.paged) == 1 and len(runner.manager.states) == 1
+        got = replay(runner, steps, seqs)
+        for rid in seqs:
+            scale = float(want[rid].abs().max())
+            err = (got[rid] - want[rid]).abs().max() / scale
+            assert err < 2e-4, (rid, float(err))
+        assert runner.manager.paged[0].pool.num_free == 40
+    # with a window, a long request holds only the pages the window covers
+    runner = ModelRunner(model, page_size=8, num_pages=40, max_num_seqs=4)
+    replay(runner, [{"step": 0, "entries": [{"id": "r2", "tokens": seqs["r2"], "want": []}], "end": []}],
+           {"r2": seqs["r2"]})
+    held = sum(p >= 0 for p in runner.manager.block_table("r2", 0))
+    assert held <= 24 // 8 + 2 < len(runner.manager.block_table("r2", 0))

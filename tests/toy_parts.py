@@ -1,0 +1,168 @@
+"""Parts defined by the tests, in plain torch, registered like any other part:
+they show that a mixer with state of its own, another feed-forward, norm,
+position scheme or whole architecture needs no change to the package's files.
+They are toys, not a model of anyone's."""
+import torch
+
+from pytriton_llama_amd.config.registry import register_model
+from pytriton_llama_amd.models import CausalLM, LayerCall
+from pytriton_llama_amd.parts import (ParamSource, Part, StateSpec, build_part, place, register_part)
+
+
+@register_part("embedding", "toy_embedding")
+class ToyEmbedding(Part):
+    def __init__(self, vocab_size, hidden_size):
+        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+
+    def param_sources(self):
+        return [ParamSource("weight", (self.vocab_size, self.hidden_size))]
+
+    def load(self, tensors, dtype, device):
+        self.weight = place(tensors["weight"], "matrix", dtype, device)
+
+    def forward(self, ids):
+        return self.weight[ids.long()]
+
+
+@register_part("norm", "toy_meannorm")
+class ToyMeanNorm(Part):
+    """Subtracts the mean: another norm, with the same interface."""
+
+    def __init__(self, size):
+        self.size = size
+
+    def forward(self, x, residual):
+        s = x if residual is None else x + residual
+        return s - s.mean(-1, keepdim=True), s
+
+
+@register_part("mixer", "toy_decay_state")
+class ToyDecayState(Part):
+    """s_t = decay * s_{t-1} + x_t W^T, y_t = s_t: a mixer whose memory is one
+    vector per request (no keys, no pages). It starts from the request's state
+    slot and writes it back, so any cutting of a sequence gives the same y."""
+
+    def __init__(self, hidden_size, decay):
+        self.hidden_size, self.decay = hidden_size, decay
+
+    def cache_spec(self):
+        return StateSpec((self.hidden_size,), torch.float32)
+
+    def param_sources(self):
+        return [ParamSource("w", (self.hidden_size, self.hidden_size))]
+
+    def load(self, tensors, dtype, device):
+        self.w = place(tensors["w"], "matrix", dtype, device)
+
+    def forward(self, x, ctx, cache):
+        u = (x.float() @ self.w.float().T)
+        y = torch.empty_like(u)
+        starts = ctx.q_start.tolist()
+        slots = ctx.state_slots.tolist()
+        for i, slot in enumerate(slots):
+            s = cache.state[slot].clone()
+            for t in range(starts[i], starts[i + 1]):
+                s = self.decay * s + u[t]
+                y[t] = s
+            if cache.writable:
+                cache.state[slot] = s
+        return y.to(x.dtype)
+
+
+@register_part("feed_forward", "toy_relu")
+class ToyRelu(Part):
+    def __init__(self, hidden_size, inner):
+        self.hidden_size, self.inner = hidden_size, inner
+
+    def param_sources(self):
+        return [ParamSource("w1", (self.inner, self.hidden_size)),
+                ParamSource("w2", (self.hidden_size, self.inner))]
+
+    def load(self, tensors, dtype, device):
+        self.w1 = place(tensors["w1"], "matrix", dtype, device)
+        self.w2 = place(tensors["w2"], "matrix", dtype, device)
+
+    def forward(self, x):
+        return torch.relu(x @ self.w1.T) @ self.w2.T
+
+
+@register_part("head", "toy_head")
+class ToyHead(Part):
+    def __init__(self, vocab_size, hidden_size):
+        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+
+    def param_sources(self):
+        return [ParamSource("weight", (self.vocab_size, self.hidden_size))]
+
+    def load(self, tensors, dtype, device):
+        self.weight = place(tensors["weight"], "matrix", dtype, device)
+
+    def forward(self, x):
+        return x.float() @ self.weight.float().T
+
+
+class ToyConfig:
+    def __init__(self, d):
+        self.__dict__.update(d)
+        self.initializer_range = d.get("initializer_range", 0.3)
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d)
+
+
+def build_toy(cfg: ToyConfig) -> CausalLM:
+    """layers: list of "state" / "attention" names; the run order is given by the
+    config too (it may name a layer twice)."""
+    H, V = cfg.hidden_size, cfg.vocab_size
+    emb = build_part("embedding", "toy_embedding", vocab_size=V, hidden_size=H)
+    blocks, prefixes = [], [("emb.", emb)]
+    for i, kind in enumerate(cfg.layers):
+        if kind == "state":
+            mixer = build_part("mixer", "toy_decay_state", hidden_size=H, decay=cfg.decay)
+        else:
+            pos = build_part("position", "rotary", head_dim=cfg.head_dim, theta=100.0)
+            mixer = build_part("mixer", "paged_attention", hidden_size=H, num_heads=cfg.heads,
+                               num_kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, position=pos,
+                               window=getattr(cfg, "window", None))
+        norm_name, norm_kw = (("toy_meannorm", dict(size=H)) if cfg.toy_norm
+                              else ("rmsnorm", dict(size=H, eps=1e-5)))
+        ffn = (build_part("feed_forward", "toy_relu", hidden_size=H, inner=cfg.inner) if cfg.toy_ffn
+               else build_part("feed_forward", "swiglu", hidden_size=H, intermediate_size=cfg.inner))
+        b = build_part("block", "prenorm", input_norm=build_part("norm", norm_name, **norm_kw),
+                       mixer=mixer, post_norm=build_part("norm", norm_name, **norm_kw), feed_forward=ffn)
+        blocks.append(b)
+        for role, part in b.children().items():
+            prefixes.append((f"l{i}.{role}.", part))
+    final = build_part("norm", "toy_meannorm", size=H) if cfg.toy_norm else \
+        build_part("norm", "rmsnorm", size=H, eps=1e-5)
+    head = build_part("head", "toy_head", vocab_size=V, hidden_size=H)
+    prefixes += [("final.", final), ("head.", head)]
+    order = getattr(cfg, "order", None) or list(range(len(blocks)))
+    # every call gets a cache layer of its own, so a block that runs twice keeps two memories
+    cache_layers = [blocks[b].cache_spec() for b in order]
+    schedule = [LayerCall(b, i) for i, b in enumerate(order)]
+    return CausalLM(cfg, emb, blocks, final, head, cache_layers, schedule, prefixes)
+
+
+register_model("ToyStateLM", ToyConfig, build_toy)
+
+
+def toy_plain_forward(model, token_ids):
+    """Whole-sequence logits of an all-toy model (state mixers only), no cache."""
+    x = model.embedding.weight[torch.as_tensor(token_ids)].float()
+    h, residual = x, None
+    for call in model.schedule:
+        b = model.blocks[call.block]
+        h, residual = b.input_norm.forward(h, residual)
+        u = h @ b.mixer.w.float().T
+        s = torch.zeros(u.shape[1])
+        ys = []
+        for t in range(u.shape[0]):
+            s = b.mixer.decay * s + u[t]
+            ys.append(s)
+        h = torch.stack(ys)
+        h, residual = b.post_norm.forward(h, residual)
+        h = b.feed_forward.forward(h)
+    h, _ = model.final_norm.forward(h, residual)
+    return model.head.forward(h)
