@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at Llama-3.2-1B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole engine (schedule, model step over the
+paged cache, sampling, bookkeeping) for a batch of requests whose prompts are
+already in the cache. The default run: random weights N(0, 0.02) of the 1B
+shape, batch 8, 2,048-token prompts of seeded uniform-random token ids, greedy
+sampling, EOS ignored. One JSON line is printed: decoded tokens a second at
+batch 8, the prefill of one 2,048-token prompt, the decode step's HBM roofline
+and the decode rates at batch 1 and 64.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+LLAMA_1B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 16, "hidden_size": 2048, "num_attention_heads": 32,
+    "num_key_value_heads": 8, "head_dim": 64, "intermediate_size": 8192, "vocab_size": 128256,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+    "max_position_embeddings": 131072, "rms_norm_eps": 1e-5, "tie_word_embeddings": True,
+    "torch_dtype": "bfloat16", "hidden_act": "silu", "initializer_range": 0.02,
+}
+
+
+def log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def model_numbers(cfg, dtype_bytes):
+    L, H, I, V = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    Hq, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    layer_params = (Hq + 2 * Hkv) * D * H + H * Hq * D + 3 * I * H
+    return {
+        "layer_params": layer_params,
+        "weight_bytes": (L * (layer_params + 2 * H) + V * H + H) * dtype_bytes,   # every weight a step uses
+        "kv_bytes_per_token": 2 * L * Hkv * D * dtype_bytes,
+        "linear_flops_per_token": 2 * L * layer_params,
+        "attn_flops": lambda S: L * 4 * D * Hq * S * (S + 1) // 2,              # causal, one prompt
+        "head_flops_per_row": 2 * V * H,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the 1B shape has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--points", default="1,64", help="other batch sizes to report, '' for none")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
+        return 2
+
+    import torch
+    from pytriton_llama_amd.config import EngineConfig
+    from pytriton_llama_amd.engine import Engine, SamplingParams
+
+    cfg = dict(LLAMA_1B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    dbytes = 2 if short == "bf16" else 4
+    nums = model_numbers(cfg, dbytes)
+    point_batches = [int(x) for x in args.points.split(",") if x]
+    max_batch = max([args.batch] + point_batches)
+    K, W, S = args.steps, args.warmup, args.prompt_len
+    page = 16
+    # requests whose prompt is in first go on decoding while the others' prompts are computed
+    slack = max_batch * -(-S // max(S, 2048)) + 8
+    per_req_pages = -(-(S + W + K + slack) // page)
+    ec = EngineConfig(dtype=args.dtype, page_size=page, num_pages=per_req_pages * max_batch + 8,
+                      max_num_seqs=max_batch, max_num_batched_tokens=max(S, 2048),
+                      max_model_len=S + W + K + slack, seed=0)
+    t0 = time.time()
+    log(f"building the {cfg['num_hidden_layers']}-layer 1B-shape model with random weights ({args.dtype})")
+    engine = Engine(cfg, ec, random_seed=0)
+    log(f"model ready in {time.time() - t0:.1f}s")
+    g = torch.Generator().manual_seed(1234)
+
+    def prompts(n):
+        return [torch.randint(0, cfg["vocab_size"], (S,), generator=g).tolist() for _ in range(n)]
+
+    def sync():
+        torch.cuda.synchronize()
+
+    # ---- prefill of one 2,048-token prompt --------------------------------------
+    prefill = None
+    if not args.no_prefill:
+        times = []
+        for i in range(4):
+            rid = engine.add_request(prompts(1)[0], SamplingParams(temperature=0.0, max_new_tokens=1,
+                                                                    ignore_eos=True))
+            sync()
+            t = time.perf_counter()
+            engine.step()                       # the whole prompt in one step, first token sampled
+            sync()
+            times.append(time.perf_counter() - t)
+            engine.requests.pop(rid, None)
+            assert not engine.has_work
+        best = min(times[1:])
+        flops = nums["linear_flops_per_token"] * S + nums["attn_flops"](S) + nums["head_flops_per_row"]
+        prefill = {"value": round(S / best, 1), "tokens": S, "ms": round(best * 1e3, 3),
+                   "frac": round(flops / best / PEAK_FLOPS[short], 4)}
+        log(f"prefill {S} tokens: {best * 1e3:.2f} ms ({S / best:.0f} tok/s)")
+
+    # ---- decode ---------------------------------------------------------------------
+    def decode_rate(batch, steps, warmup):
+        sp = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + slack - 4, ignore_eos=True)
+        ids = [engine.add_request(p, sp) for p in prompts(batch)]
+        while any(engine.requests[i].num_computed < S for i in ids):
+            engine.step()                       # prompts go in, portion by portion
+        for _ in range(warmup):
+            engine.step()
+        sync()
+        t = time.perf_counter()
+        produced = 0
+        for _ in range(steps):
+            produced += len(engine.step())
+        sync()
+        dt = time.perf_counter() - t
+        assert produced == batch * steps, (produced, batch, steps)
+        ctx = [engine.requests[i].num_computed for i in ids]
+        for i in ids:
+            engine.scheduler.abort(engine.requests.pop(i))
+        assert not engine.has_work
+        mean_ctx = sum(ctx) / len(ctx) - steps / 2.0
+        return batch * steps / dt, dt / steps, mean_ctx
+
+    rate, step_s, mean_ctx = decode_rate(args.batch, K, W)
+    log(f"decode batch {args.batch}: {rate:.0f} tok/s, {step_s * 1e3:.3f} ms/step")
+    bytes_step = nums["weight_bytes"] + args.batch * mean_ctx * nums["kv_bytes_per_token"]
+    achieved = bytes_step / step_s / 1e9
+    points = {}
+    for b in point_batches:
+        r, st, _ = decode_rate(b, max(16, K // 2), max(4, W // 2))
+        points[f"decode_b{b}"] = round(r, 1)
+        log(f"decode batch {b}: {r:.0f} tok/s, {st * 1e3:.3f} ms/step")
+
+    out = {
+        "metric": f"decode tokens/s, Llama-3.2-1B shape, batch {args.batch}, {S}-token prompts",
+        "value": round(rate, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": short, "data": "synthetic",
+        "config": {
+            "model": "Llama-3.2-1B shape, random weights N(0,0.02)", "layers": cfg["num_hidden_layers"],
+            "layers_of_full_model": full_layers, "hidden_size": cfg["hidden_size"],
+            "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["head_dim"], "intermediate_size": cfg["intermediate_size"],
+            "vocab_size": cfg["vocab_size"], "tied_embeddings": True, "rope": "llama3 factor 32",
+            "global_batch": args.batch, "seq_len": S, "context_at_timing": round(mean_ctx),
+            "page_size": page, "kv_dtype": short, "sampling": "greedy", "parallelism": "single GPU",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+    }
+    if prefill is not None:
+        out["prefill"] = prefill
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
