@@ -177,3 +177,506 @@ extern "C" int ptl_attention_generic(void* out, long out_stride, const void* q, 
 #undef GO
   return PTL_ERR_ARG;
 }
+
+// ===========================================================================
+// ptl_attention_decode: one query token per sequence against its pages, the
+// keys split over several workgroups (flash-decoding; the reference's stage 1
+// and stage 2 are lite_llama/kernels/flashdecoding.py:22-131 and :171-231:
+// every partition emits its accumulator with its running max and denominator,
+// the merge weighs them by exp(max_p - max)).
+//
+// Grid (sequence, kv head x head group, split). A workgroup of four waves
+// serves up to GT query heads that share one kv head, so every key and value
+// is read once for all of them. A wave reads 64/LPK keys per turn: LPK lanes
+// share a key, each lane owns 16 elements of the head dimension of that key
+// and of the matching value, for all heads. Every key slot (LPK lanes) keeps
+// an online softmax of its own; slots, waves and splits are merged at the end.
+// Needs D % 16 == 0. Float32 math throughout.
+// ===========================================================================
+#define DEC_CHUNK 16
+
+template <typename T> struct Chunk16 { float v[DEC_CHUNK]; };
+
+template <typename T>
+__device__ __forceinline__ void load_chunk(const T* __restrict__ p, float* out);
+
+template <>
+__device__ __forceinline__ void load_chunk<float>(const float* __restrict__ p, float* out) {
+  const float4* p4 = reinterpret_cast<const float4*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float4 x = p4[i];
+    out[4 * i] = x.x; out[4 * i + 1] = x.y; out[4 * i + 2] = x.z; out[4 * i + 3] = x.w;
+  }
+}
+
+template <>
+__device__ __forceinline__ void load_chunk<bf16_t>(const bf16_t* __restrict__ p, float* out) {
+  const uint4* p4 = reinterpret_cast<const uint4*>(p);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint4 x = p4[i];
+    const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      out[8 * i + 2 * j] = __uint_as_float(w[j] << 16);
+      out[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  }
+}
+
+template <typename T, int GT, int LPK>
+__global__ void __launch_bounds__(256)
+attn_decode_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q, long q_stride,
+                   const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
+                   const int32_t* __restrict__ block_table, int bt_stride,
+                   float* __restrict__ part_acc, float* __restrict__ part_ml,
+                   int Hq, int Hkv, int D, int page_size, int window, float scale,
+                   int num_splits, int groups_per_kv) {
+  constexpr int KPW = 64 / LPK;           // keys a wave reads per turn
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int seq = blockIdx.x;
+  const int kvh = blockIdx.y / groups_per_kv;
+  const int hg = blockIdx.y - kvh * groups_per_kv;
+  const int split = blockIdx.z;
+  const int G = Hq / Hkv;
+  const int head0 = kvh * G + hg * GT;      // first query head of this workgroup
+  const int nheads = min(GT, G - hg * GT);
+  const int row = q_start[seq];
+  const int ctx = ctx_len[seq];
+  const int k_lo = window > 0 ? max(0, ctx - window) : 0;
+  const int span = ctx - k_lo;
+  const int tile = 4 * KPW;
+  const int per_split = ((span + num_splits - 1) / num_splits + tile - 1) / tile * tile;
+  const int k_begin = k_lo + split * per_split;
+  const int k_end = min(ctx, k_begin + per_split);
+  const int32_t* bt = block_table + (size_t)seq * bt_stride;
+
+  const int c = lane % LPK;                 // which 16 elements of the head this lane owns
+  const int ks = lane / LPK;                // key slot within the wave
+  const bool active = c * DEC_CHUNK < D;
+
+  float qf[GT][DEC_CHUNK];
+#pragma unroll
+  for (int h = 0; h < GT; ++h) {
+    if (h < nheads && active) {
+      load_chunk<T>(q + (size_t)row * q_stride + (size_t)(head0 + h) * D + c * DEC_CHUNK, qf[h]);
+#pragma unroll
+      for (int j = 0; j < DEC_CHUNK; ++j) qf[h][j] *= scale;
+    } else {
+#pragma unroll
+      for (int j = 0; j < DEC_CHUNK; ++j) qf[h][j] = 0.f;
+    }
+  }
+  float m[GT], l[GT], acc[GT][DEC_CHUNK];
+#pragma unroll
+  for (int h = 0; h < GT; ++h) {
+    m[h] = -INFINITY; l[h] = 0.f;
+#pragma unroll
+    for (int j = 0; j < DEC_CHUNK; ++j) acc[h][j] = 0.f;
+  }
+
+  for (int kb = k_begin + wave * KPW; kb < k_end; kb += tile) {
+    const int kp = kb + ks;
+    const bool valid = kp < k_end;
+    float kf[DEC_CHUNK], vf[DEC_CHUNK];
+    if (valid && active) {
+      const int page = bt[kp / page_size];
+      const size_t idx = (((size_t)page * Hkv + kvh) * page_size + (kp % page_size)) * D + c * DEC_CHUNK;
+      load_chunk<T>(k_cache + idx, kf);
+      load_chunk<T>(v_cache + idx, vf);
+    } else {
+#pragma unroll
+      for (int j = 0; j < DEC_CHUNK; ++j) { kf[j] = 0.f; vf[j] = 0.f; }
+    }
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+      float s = 0.f;
+#pragma unroll
+      for (int j = 0; j < DEC_CHUNK; ++j) s = fmaf(qf[h][j], kf[j], s);
+#pragma unroll
+      for (int o = 1; o < LPK; o <<= 1) s += __shfl_xor(s, o, 64);
+      if (valid) {
+        if (s > m[h]) {
+          const float alpha = expf(m[h] - s);     // exp(-inf) = 0 at the first key
+          l[h] *= alpha;
+#pragma unroll
+          for (int j = 0; j < DEC_CHUNK; ++j) acc[h][j] *= alpha;
+          m[h] = s;
+        }
+        const float p = expf(s - m[h]);
+        l[h] += p;
+#pragma unroll
+        for (int j = 0; j < DEC_CHUNK; ++j) acc[h][j] = fmaf(p, vf[j], acc[h][j]);
+      }
+    }
+  }
+
+  // merge the key slots of the wave
+#pragma unroll
+  for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+      const float mo = __shfl_xor(m[h], o, 64);
+      const float lo = __shfl_xor(l[h], o, 64);
+      const float mn = fmaxf(m[h], mo);
+      const float ms = mn == -INFINITY ? 0.f : mn;
+      const float a = expf(m[h] - ms), b = expf(mo - ms);
+      l[h] = l[h] * a + lo * b;
+#pragma unroll
+      for (int j = 0; j < DEC_CHUNK; ++j)
+        acc[h][j] = acc[h][j] * a + __shfl_xor(acc[h][j], o, 64) * b;
+      m[h] = mn;
+    }
+  }
+
+  // merge the four waves through LDS
+  extern __shared__ float lds[];
+  float* w_acc = lds;                         // [4][GT][D]
+  float* w_ml = lds + 4 * GT * D;             // [4][GT][2]
+  if (ks == 0 && active) {
+#pragma unroll
+    for (int h = 0; h < GT; ++h) {
+#pragma unroll
+      for (int j = 0; j < DEC_CHUNK; ++j) w_acc[(wave * GT + h) * D + c * DEC_CHUNK + j] = acc[h][j];
+      if (c == 0) { w_ml[(wave * GT + h) * 2] = m[h]; w_ml[(wave * GT + h) * 2 + 1] = l[h]; }
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < nheads * D; i += 256) {
+    const int h = i / D, d = i - h * D;
+    float mn = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mn = fmaxf(mn, w_ml[(w * GT + h) * 2]);
+    const float ms = mn == -INFINITY ? 0.f : mn;
+    float ll = 0.f, a = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = expf(w_ml[(w * GT + h) * 2] - ms);
+      ll += w_ml[(w * GT + h) * 2 + 1] * f;
+      a += w_acc[(w * GT + h) * D + d] * f;
+    }
+    const int head = head0 + h;
+    if (num_splits == 1) {
+      out[(size_t)row * out_stride + (size_t)head * D + d] = from_float<T>(ll > 0.f ? a / ll : 0.f);
+    } else {
+      const size_t pi = ((size_t)seq * Hq + head) * num_splits + split;
+      part_acc[pi * D + d] = a;
+      if (d == 0) { part_ml[pi * 2] = mn; part_ml[pi * 2 + 1] = ll; }
+    }
+  }
+}
+
+template <typename T>
+__global__ void attn_decode_merge_kernel(T* __restrict__ out, long out_stride,
+                                         const int32_t* __restrict__ q_start,
+                                         const float* __restrict__ part_acc,
+                                         const float* __restrict__ part_ml,
+                                         int Hq, int D, int num_splits) {
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const size_t base = ((size_t)seq * Hq + head) * num_splits;
+  float mn = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) mn = fmaxf(mn, part_ml[(base + s) * 2]);
+  const float ms = mn == -INFINITY ? 0.f : mn;
+  float ll = 0.f;
+  for (int s = 0; s < num_splits; ++s) ll += part_ml[(base + s) * 2 + 1] * expf(part_ml[(base + s) * 2] - ms);
+  const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+  const int row = q_start[seq];
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < num_splits; ++s)
+      a += part_acc[(base + s) * D + d] * expf(part_ml[(base + s) * 2] - ms);
+    out[(size_t)row * out_stride + (size_t)head * D + d] = from_float<T>(a * inv);
+  }
+}
+
+template <typename T, int LPK>
+static int launch_decode(void* out, long out_stride, const void* q, long q_stride,
+                         const void* k_cache, const void* v_cache, const int32_t* q_start,
+                         const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
+                         float* part_acc, float* part_ml, int n_seq, int Hq, int Hkv, int D,
+                         int page_size, int window, float scale, int num_splits, hipStream_t stream) {
+  constexpr int GT = 4;
+  const int G = Hq / Hkv;
+  const int groups = (G + GT - 1) / GT;
+  dim3 grid(n_seq, Hkv * groups, num_splits);
+  const size_t lds = (size_t)(4 * GT * D + 4 * GT * 2) * sizeof(float);
+  attn_decode_kernel<T, GT, LPK><<<grid, 256, lds, stream>>>(
+      (T*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, q_start,
+      ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv, D, page_size, window, scale,
+      num_splits, groups);
+  if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
+  if (num_splits > 1) {
+    dim3 mgrid(n_seq, Hq);
+    attn_decode_merge_kernel<T><<<mgrid, 64, 0, stream>>>((T*)out, out_stride, q_start, part_acc,
+                                                         part_ml, Hq, D, num_splits);
+  }
+  return ptl_launch_status();
+}
+
+// Sequences 0..n_seq-1 of the tables each bring one query token (row q_start[s]).
+// part_acc [n_seq, Hq, num_splits, D] and part_ml [n_seq, Hq, num_splits, 2] are
+// float32 workspaces of the caller (unused when num_splits == 1).
+extern "C" int ptl_attention_decode(void* out, long out_stride, const void* q, long q_stride,
+                                    const void* k_cache, const void* v_cache,
+                                    const int32_t* q_start, const int32_t* ctx_len,
+                                    const int32_t* block_table, int bt_stride, float* part_acc,
+                                    float* part_ml, int n_seq, int Hq, int Hkv, int D, int page_size,
+                                    int window, float scale, int num_splits, int dtype,
+                                    hipStream_t stream) {
+  if (n_seq <= 0) return PTL_OK;
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || D % 16 || D > 256 || page_size <= 0 ||
+      num_splits < 1 || num_splits > 65535 || (num_splits > 1 && (!part_acc || !part_ml)))
+    return PTL_ERR_ARG;
+  const int chunks = D / 16;
+  int lpk = 1;
+  while (lpk < chunks) lpk <<= 1;
+#define GO(T, L) launch_decode<T, L>(out, out_stride, q, q_stride, k_cache, v_cache, q_start,      \
+                                     ctx_len, block_table, bt_stride, part_acc, part_ml, n_seq,    \
+                                     Hq, Hkv, D, page_size, window, scale, num_splits, stream)
+#define BY_LPK(T)                                                                                  \
+  switch (lpk) {                                                                                   \
+    case 1: return GO(T, 1);                                                                       \
+    case 2: return GO(T, 2);                                                                       \
+    case 4: return GO(T, 4);                                                                       \
+    case 8: return GO(T, 8);                                                                       \
+    default: return GO(T, 16);                                                                     \
+  }
+  if (dtype == PTL_DTYPE_F32) { BY_LPK(float) }
+  if (dtype == PTL_DTYPE_BF16) { BY_LPK(bf16_t) }
+#undef BY_LPK
+#undef GO
+  return PTL_ERR_ARG;
+}
+
+// ===========================================================================
+// ptl_attention_prefill_mfma: bfloat16 prompt portions on the matrix cores.
+//
+// A workgroup of four waves takes 64 query rows of one head (16 per wave) and
+// walks the sequence's keys in tiles of 64, through LDS. Both products are
+// computed transposed so that the scores leave the first MFMA in the register
+// layout the second one wants, without a shuffle:
+//   S^T[key, query] = K[key, :] . Q[query, :]      (A = K tile, B = Q^T)
+//   O^T[d, query]  += V^T[d, key] . P^T[key, query] (A = V^T tile, B = P^T)
+// with v_mfma_f32_16x16x32_bf16: a lane holds 8 consecutive k-values of row
+// (lane % 16), k-group (lane / 16); the result tile holds rows 4*(lane/16)+i,
+// column lane % 16. V^T is made when the value tile is written to LDS, with the
+// groups of four keys XOR-swizzled by the row so that reads and writes spread
+// over the banks. Softmax is the online one of
+// lite_llama/kernels/flashattentionv2.py:10-61 in base 2 (scale * log2 e folded
+// into the scores, exp2), float32 max / denominator / accumulator; P is rounded
+// to bfloat16 for the second product as there (:55).
+// Needs D % 32 == 0, D <= 128.
+// ===========================================================================
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+#define PF_BM 64
+#define PF_BN 64
+
+union Frag8 {
+  uint4 u;
+  uint2 h[2];
+  bf16x8_t v;
+};
+
+template <int NDT>
+__global__ void __launch_bounds__(256)
+attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
+                         long q_stride, const bf16_t* __restrict__ k_cache,
+                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ q_start,
+                         const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ block_table,
+                         int bt_stride, const int32_t* __restrict__ work_seq,
+                         const int32_t* __restrict__ work_qoff, int Hq, int Hkv, int page_size,
+                         int window, float scale_log2) {
+  constexpr int D = 32 * NDT;
+  constexpr int KS = D + 8;            // row stride of the key tile, in elements
+  constexpr int CPR = D / 8;           // 16-byte chunks per row
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_BN * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t Vt[D * PF_BN];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ln = lane & 15, lg = lane >> 4;
+  const int head = blockIdx.y;
+  const int seq = work_seq[blockIdx.x];
+  const int qoff = work_qoff[blockIdx.x];
+  const int qs = q_start[seq];
+  const int qlen = q_start[seq + 1] - qs;
+  const int ctx = ctx_len[seq];
+  const int cached = ctx - qlen;
+  const int rows = min(PF_BM, qlen - qoff);
+  if (rows <= 0) return;
+  const int kvh = head / (Hq / Hkv);
+  const int32_t* bt = block_table + (size_t)seq * bt_stride;
+
+  const int my_row = 16 * wave + ln;
+  const bool row_ok = my_row < rows;
+  const int qrow = row_ok ? my_row : 0;       // rows past the end repeat row 0; never stored
+  const int first_q = cached + qoff;
+  const int qpos = first_q + qrow;
+  const int wave_min_q = (16 * wave < rows) ? first_q + 16 * wave : first_q;
+
+  Frag8 qf[NDT];
+  {
+    const bf16_t* qp = q + (size_t)(qs + qoff + qrow) * q_stride + (size_t)head * D + 8 * lg;
+#pragma unroll
+    for (int kk = 0; kk < NDT; ++kk) qf[kk].u = *reinterpret_cast<const uint4*>(qp + 32 * kk);
+  }
+  f32x4_t o[2 * NDT];
+#pragma unroll
+  for (int t = 0; t < 2 * NDT; ++t) o[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_part = 0.f;
+
+  const int k_end = min(ctx, first_q + rows);
+  const int k_lo = window > 0 ? max(0, first_q - window + 1) : 0;
+  const int k_begin = (k_lo / PF_BN) * PF_BN;
+
+  for (int k0 = k_begin; k0 < k_end; k0 += PF_BN) {
+    __syncthreads();
+    for (int c = tid; c < PF_BN * CPR; c += 256) {
+      const int r = c / CPR, cc = c - r * CPR;
+      const int kp = k0 + r;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (kp >= k_lo && kp < k_end) {
+        const int page = bt[kp / page_size];
+        if (page >= 0)
+          val = *reinterpret_cast<const uint4*>(
+              k_cache + (((size_t)page * Hkv + kvh) * page_size + (kp % page_size)) * D + cc * 8);
+      }
+      *reinterpret_cast<uint4*>(Ks + r * KS + cc * 8) = val;
+    }
+    for (int c = tid; c < PF_BN * CPR; c += 256) {
+      const int key = c & (PF_BN - 1), dc = c / PF_BN;
+      const int kp = k0 + key;
+      union { uint4 u; bf16_t e[8]; } val;
+      val.u = make_uint4(0, 0, 0, 0);
+      if (kp >= k_lo && kp < k_end) {
+        const int page = bt[kp / page_size];
+        if (page >= 0)
+          val.u = *reinterpret_cast<const uint4*>(
+              v_cache + (((size_t)page * Hkv + kvh) * page_size + (kp % page_size)) * D + dc * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int d = dc * 8 + j;
+        Vt[d * PF_BN + ((((key >> 2) ^ (d & 15)) << 2) | (key & 3))] = val.e[j];
+      }
+    }
+    __syncthreads();
+
+    f32x4_t st[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      st[kt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NDT; ++kk) {
+        Frag8 a;
+        a.u = *reinterpret_cast<const uint4*>(Ks + (16 * kt + ln) * KS + 32 * kk + 8 * lg);
+        st[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[kk].v, st[kt], 0, 0, 0);
+      }
+    }
+    const bool need_mask = (k0 + PF_BN - 1 > wave_min_q) || (k0 + PF_BN > k_end) || window > 0;
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float s = st[kt][i] * scale_log2;
+        if (need_mask) {
+          const int key = k0 + 16 * kt + 4 * lg + i;
+          const bool vis = key <= qpos && key < k_end && (window <= 0 || key > qpos - window);
+          s = vis ? s : -INFINITY;
+        }
+        st[kt][i] = s;
+        tmax = fmaxf(tmax, s);
+      }
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    m_run = m_new;
+    l_part *= alpha;
+#pragma unroll
+    for (int t = 0; t < 2 * NDT; ++t) {
+      o[t][0] *= alpha; o[t][1] *= alpha; o[t][2] *= alpha; o[t][3] *= alpha;
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      Frag8 pb;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = __builtin_amdgcn_exp2f(st[2 * half + t][i] - m_safe);
+          l_part += p;
+          pb.v[4 * t + i] = (__bf16)p;
+        }
+      }
+#pragma unroll
+      for (int dt = 0; dt < 2 * NDT; ++dt) {
+        const int d = 16 * dt + ln;
+        const int g0 = 8 * half + lg, g1 = g0 + 4;
+        Frag8 a;
+        a.h[0] = *reinterpret_cast<const uint2*>(Vt + d * PF_BN + ((g0 ^ ln) << 2));
+        a.h[1] = *reinterpret_cast<const uint2*>(Vt + d * PF_BN + ((g1 ^ ln) << 2));
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb.v, o[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  float l = l_part + __shfl_xor(l_part, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (row_ok) {
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16_t* op = out + (size_t)(qs + qoff + my_row) * out_stride + (size_t)head * D + 4 * lg;
+#pragma unroll
+    for (int dt = 0; dt < 2 * NDT; ++dt) {
+      union { uint2 u; bf16_t e[4]; } r;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r.e[i] = float_to_bf16(o[dt][i] * inv);
+      *reinterpret_cast<uint2*>(op + 16 * dt) = r.u;
+    }
+  }
+}
+
+template <int NDT>
+static int launch_prefill_mfma(void* out, long out_stride, const void* q, long q_stride,
+                               const void* k_cache, const void* v_cache, const int32_t* q_start,
+                               const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
+                               const int32_t* work_seq, const int32_t* work_qoff, int n_work, int Hq,
+                               int Hkv, int page_size, int window, float scale, hipStream_t stream) {
+  dim3 grid(n_work, Hq);
+  attn_prefill_mfma_kernel<NDT><<<grid, 256, 0, stream>>>(
+      (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+      (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff, Hq, Hkv,
+      page_size, window, scale * 1.4426950408889634f);
+  return ptl_launch_status();
+}
+
+// work_seq / work_qoff list 64-row query blocks. bfloat16 only; q rows and the
+// output rows must be 16-byte aligned (q_stride and out_stride multiples of 8).
+extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void* q, long q_stride,
+                                          const void* k_cache, const void* v_cache,
+                                          const int32_t* q_start, const int32_t* ctx_len,
+                                          const int32_t* block_table, int bt_stride,
+                                          const int32_t* work_seq, const int32_t* work_qoff,
+                                          int n_work, int Hq, int Hkv, int D, int page_size,
+                                          int window, float scale, hipStream_t stream) {
+  if (n_work <= 0) return PTL_OK;
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D % 32 || D <= 0 || D > 128 || page_size <= 0 ||
+      Hq > 65535 || q_stride % 8 || out_stride % 4)
+    return PTL_ERR_ARG;
+#define GO(N) launch_prefill_mfma<N>(out, out_stride, q, q_stride, k_cache, v_cache, q_start,      \
+                                     ctx_len, block_table, bt_stride, work_seq, work_qoff, n_work, \
+                                     Hq, Hkv, page_size, window, scale, stream)
+  switch (D / 32) {
+    case 1: return GO(1);
+    case 2: return GO(2);
+    case 3: return GO(3);
+    default: return GO(4);
+  }
+#undef GO
+}

@@ -14,7 +14,21 @@ from typing import Hashable, List, Optional, Sequence
 
 import torch
 
-ATTN_BLOCK_ROWS = 16    # query rows per work item of the attention kernels
+GENERIC_BLOCK_ROWS = 16   # query rows per work item of the vector-FMA attention kernel
+MFMA_BLOCK_ROWS = 64      # ... of the matrix-core prefill kernel
+
+
+def work_items(q_lens, ctx_lens, first_seq: int, block_rows: int):
+    """(sequence, first row) of every block of ``block_rows`` query rows of the
+    sequences from ``first_seq`` on, the blocks with the most keys first so
+    that the long ones do not end the launch alone."""
+    items = []
+    for s in range(first_seq, len(q_lens)):
+        cached = ctx_lens[s] - q_lens[s]
+        for off in range(0, q_lens[s], block_rows):
+            items.append((cached + min(off + block_rows, q_lens[s]), s, off))
+    items.sort(key=lambda t: -t[0])
+    return [s for _, s, _ in items], [o for _, _, o in items]
 
 
 @dataclass
@@ -40,8 +54,10 @@ class StepContext:
     ctx_len: torch.Tensor          # int32 [n]: tokens of the sequence in the cache after this step
     state_slots: torch.Tensor      # int32 [n]: state slot of every sequence
     logit_rows: torch.Tensor       # int32 [R]: rows whose logits are wanted
-    work_seq: torch.Tensor         # int32 [W]: attention work items (sequence,
-    work_qoff: torch.Tensor        # int32 [W]:   first query row within it)
+    work: dict                     # name -> (sequence int32 [W], first query row int32 [W]):
+                                   # "all16": 16-row blocks of every sequence; "multi16" /
+                                   # "multi64": 16- / 64-row blocks of the sequences after the
+                                   # leading single-token ones
     groups: List[GroupContext]
     num_tokens: int
     num_seqs: int
@@ -119,11 +135,12 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
     T = len(token_ids)
     nseq = len(order)
     q_lens = [q_start[i + 1] - q_start[i] for i in range(nseq)]
-    work_seq, work_qoff = [], []
-    for s, ql in enumerate(q_lens):
-        for off in range(0, ql, ATTN_BLOCK_ROWS):
-            work_seq.append(s)
-            work_qoff.append(off)
+    num_decode = 0
+    while num_decode < nseq and q_lens[num_decode] == 1:
+        num_decode += 1
+    work = {"all16": work_items(q_lens, ctx_len, 0, GENERIC_BLOCK_ROWS),
+            "multi16": work_items(q_lens, ctx_len, num_decode, GENERIC_BLOCK_ROWS),
+            "multi64": work_items(q_lens, ctx_len, num_decode, MFMA_BLOCK_ROWS)}
     tables = []
     for g, group in enumerate(manager.paged):
         rows = [group.tables[entries[i].request] for i in order]
@@ -144,8 +161,9 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
     put("ctx_len", ctx_len)
     put("state_slots", state_slots)
     put("logit_rows", logit_rows)
-    put("work_seq", work_seq)
-    put("work_qoff", work_qoff)
+    for name, (ws, wo) in work.items():
+        put("ws_" + name, ws)
+        put("wo_" + name, wo)
     for g in range(len(manager.paged)):
         put(f"slots{g}", slots[g])
         put(f"table{g}", [p for row in tables[g] for p in row])
@@ -162,9 +180,9 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
     ctx = StepContext(
         token_ids=get("token_ids"), positions=get("positions"), q_start=get("q_start"),
         ctx_len=get("ctx_len"), state_slots=get("state_slots"), logit_rows=get("logit_rows"),
-        work_seq=get("work_seq"), work_qoff=get("work_qoff"), groups=groups,
+        work={name: (get("ws_" + name), get("wo_" + name)) for name in work}, groups=groups,
         num_tokens=T, num_seqs=nseq, num_logit_rows=len(logit_rows),
         logit_rows_are_identity=logit_rows == list(range(T)),
-        num_decode_seqs=sum(1 for q in q_lens if q == 1),
+        num_decode_seqs=num_decode,
         q_lens=q_lens, ctx_lens=ctx_len, max_q_len=max(q_lens), max_ctx_len=max(ctx_len))
     return ctx, order

@@ -217,6 +217,83 @@ def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         "attention")
 
 
+def _attention_common(out, q, k_cache, v_cache, q_start, ctx_len, block_table, what):
+    _need_gpu(out, q, k_cache, v_cache, q_start, ctx_len, block_table)
+    T, Hq, D = q.shape
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[3] != D:
+        raise KernelError(f"{what}: caches must be [pages, Hkv, page_size, D]")
+    Hkv, page_size = k_cache.shape[1], k_cache.shape[2]
+    if Hq % Hkv:
+        raise KernelError(f"{what}: {Hq} query heads are not a multiple of {Hkv} kv heads")
+    if q.stride(2) != 1 or out.stride(2) != 1 or (Hq > 1 and (q.stride(1) != D or out.stride(1) != D)):
+        raise KernelError(f"{what}: q and out need dense heads")
+    if not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
+        raise KernelError(f"{what}: q, out and the caches must share one dtype")
+    if not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError(f"{what}: caches must be contiguous")
+    _i32(q_start, "q_start")
+    _i32(ctx_len, "ctx_len")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError(f"{what}: block_table must be int32 [n, max_pages]")
+    return T, Hq, Hkv, D, page_size
+
+
+def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                     v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
+                     block_table: torch.Tensor, n_seq: int, scale: float, window: int = 0,
+                     num_splits: int = 1) -> None:
+    """Split-KV attention of the first ``n_seq`` sequences of the tables, each of
+    which brings exactly one query token (see csrc/attention.hip). Head sizes in
+    steps of 16 up to 256, float32 or bfloat16."""
+    T, Hq, Hkv, D, page_size = _attention_common(out, q, k_cache, v_cache, q_start, ctx_len,
+                                                 block_table, "attention_decode")
+    if D % 16 or D > 256:
+        raise KernelError(f"attention_decode: head size {D} is not a multiple of 16 up to 256")
+    if n_seq > ctx_len.numel() or q_start.numel() < n_seq + 1 or block_table.shape[0] < n_seq:
+        raise KernelError("attention_decode: tables are shorter than n_seq")
+    if num_splits < 1:
+        raise KernelError("attention_decode: num_splits must be >= 1")
+    part_acc = part_ml = None
+    if num_splits > 1:
+        part_acc = torch.empty((n_seq, Hq, num_splits, D), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_seq, Hq, num_splits, 2), dtype=torch.float32, device=q.device)
+    lib = library.load("attention")
+    _check(lib.ptl_attention_decode(
+        _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
+        _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
+        int(block_table.stride(0)), _ptr(part_acc), _ptr(part_ml), int(n_seq), Hq, Hkv, D, page_size,
+        int(window), ctypes.c_float(scale), int(num_splits), _dtype_code(q), _stream()),
+        "attention_decode")
+
+
+def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                           v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
+                           block_table: torch.Tensor, work_seq: torch.Tensor,
+                           work_qoff: torch.Tensor, scale: float, window: int = 0) -> None:
+    """bfloat16 attention of prompt portions on the matrix cores; the work list
+    names 64-row query blocks. Head sizes 32, 64, 96, 128."""
+    T, Hq, Hkv, D, page_size = _attention_common(out, q, k_cache, v_cache, q_start, ctx_len,
+                                                 block_table, "attention_prefill_mfma")
+    if q.dtype != torch.bfloat16:
+        raise KernelError("attention_prefill_mfma: bfloat16 only")
+    if D % 32 or D > 128:
+        raise KernelError(f"attention_prefill_mfma: head size {D} is not 32, 64, 96 or 128")
+    _need_gpu(work_seq, work_qoff)
+    _i32(work_seq, "work_seq")
+    _i32(work_qoff, "work_qoff")
+    if work_seq.numel() != work_qoff.numel():
+        raise KernelError("attention_prefill_mfma: inconsistent work list")
+    if q.stride(0) % 8 or out.stride(0) % 4 or q.data_ptr() % 16 or out.data_ptr() % 8:
+        raise KernelError("attention_prefill_mfma: q rows must be 16-byte aligned, out rows 8-byte")
+    lib = library.load("attention")
+    _check(lib.ptl_attention_prefill_mfma(
+        _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
+        _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
+        int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), int(work_seq.numel()),
+        Hq, Hkv, D, page_size, int(window), ctypes.c_float(scale), _stream()),
+        "attention_prefill_mfma")
+
+
 def argmax(logits: torch.Tensor) -> torch.Tensor:
     """Greedy token per row of float32 logits [R, V]; ties go to the lowest id."""
     _need_gpu(logits)

@@ -39,6 +39,7 @@ class PagedAttention(Part):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.window = int(window) if window else None
         self.names = (q_name, k_name, v_name, o_name)
+        self.force_decode_splits = 0        # tests set it to try other splits
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim
         self.qkv: Optional[torch.Tensor] = None
@@ -83,7 +84,42 @@ class PagedAttention(Part):
                        group.slots if cache.writable else None, cache.k, cache.v,
                        cache.page_size)
         out = torch.empty((T, Hq, D), dtype=x.dtype, device=x.device)
-        ops.attention_generic(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
-                              group.block_table, ctx.work_seq, ctx.work_qoff, self.scale,
-                              self.window or 0)
+        self.attend(out, q, cache, ctx, group)
         return linear(out.view(T, Hq * D), self.o)
+
+    # ---- which kernel takes which sequences --------------------------------------
+    def decode_splits(self, ctx, n_dec: int) -> int:
+        """How many workgroups share one sequence's keys: enough to fill the 256
+        CUs a few times over, never finer than one turn of a workgroup."""
+        if self.force_decode_splits:
+            return self.force_decode_splits
+        D = self.head_dim
+        lpk = 1
+        while lpk * 16 < D:
+            lpk <<= 1
+        tile = 256 // lpk
+        groups = self.num_kv_heads * (-(-(self.num_heads // self.num_kv_heads) // 4))
+        span = max(ctx.ctx_lens[:n_dec])
+        if self.window:
+            span = min(span, self.window)
+        want = -(-1024 // max(1, n_dec * groups))
+        return max(1, min(want, -(-span // tile), 64))
+
+    def attend(self, out, q, cache, ctx, group) -> None:
+        D, window = self.head_dim, self.window or 0
+        n_dec = ctx.num_decode_seqs if D % 16 == 0 else 0
+        if n_dec:
+            ops.attention_decode(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
+                                 group.block_table, n_dec, self.scale, window,
+                                 self.decode_splits(ctx, n_dec))
+        if n_dec == ctx.num_seqs:
+            return
+        if q.dtype == torch.bfloat16 and D % 32 == 0 and D <= 128:
+            ws, wo = ctx.work["multi64"]
+            ops.attention_prefill_mfma(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
+                                       group.block_table, ws, wo, self.scale, window)
+        else:
+            ws, wo = ctx.work["multi16"] if n_dec else ctx.work["all16"]
+            ops.attention_generic(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
+                                  group.block_table, ws, wo, self.scale, window)
+

@@ -148,7 +148,8 @@ def _paged_setup(seq_lens, q_lens, Hkv, D, P, dtype, seed, shuffle=True):
     return kc, vc, bt, dense_k, dense_v
 
 
-def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=0, boost=None):
+def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=0, boost=None,
+                    kernel="generic", splits=1):
     kc, vc, bt, dk, dv = _paged_setup(seq_lens, q_lens, Hkv, D, P, dtype, seed)
     g = torch.Generator().manual_seed(seed + 100)
     T = sum(q_lens)
@@ -158,17 +159,30 @@ def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=
     q_start = [0]
     for ql in q_lens:
         q_start.append(q_start[-1] + ql)
+    rows = 64 if kernel == "mfma" else 16
     work_seq, work_qoff = [], []
     for s, ql in enumerate(q_lens):
-        for off in range(0, ql, 16):
+        for off in range(0, ql, rows):
             work_seq.append(s)
             work_qoff.append(off)
     dev = "cuda"
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
     out = torch.zeros(T, Hq, D, dtype=dtype, device=dev)
     scale = 1.0 / math.sqrt(D)
-    ops.attention_generic(out, q.to(dev), kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
-                          bt.to(dev), i32(work_seq), i32(work_qoff), scale, window)
+    # q as the engine has it: a slice of a wider projection buffer
+    wide = torch.zeros(T, Hq * D + 64, dtype=dtype, device=dev)
+    wide[:, :Hq * D] = q.to(dev).view(T, Hq * D)
+    qd = wide[:, :Hq * D].view(T, Hq, D)
+    if kernel == "generic":
+        ops.attention_generic(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
+                              bt.to(dev), i32(work_seq), i32(work_qoff), scale, window)
+    elif kernel == "mfma":
+        ops.attention_prefill_mfma(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
+                                   bt.to(dev), i32(work_seq), i32(work_qoff), scale, window)
+    else:
+        assert all(ql == 1 for ql in q_lens)
+        ops.attention_decode(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
+                             bt.to(dev), len(q_lens), scale, window, splits)
     # plain: full causal attention over the sequence, rows of the portion kept
     for i, (s, ql) in enumerate(zip(seq_lens, q_lens)):
         full_q = torch.zeros(s, Hq, D)
@@ -189,6 +203,56 @@ def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=
 ])
 def test_attention_generic(ops, dtype, case):
     _attention_case(ops, dtype, **case)
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("case", [
+    dict(seq_lens=[37, 5, 130, 1], Hq=8, Hkv=2, D=48, P=4),         # 3 lanes of 4 per key
+    dict(seq_lens=[300, 64, 65], Hq=4, Hkv=4, D=64, P=16),          # MHA
+    dict(seq_lens=[100, 257], Hq=16, Hkv=2, D=16, P=8),             # 8 heads a kv head: two groups
+    dict(seq_lens=[90, 33], Hq=3, Hkv=1, D=128, P=16),              # 3 heads of a tile of 4
+    dict(seq_lens=[70], Hq=2, Hkv=1, D=256, P=5),                   # widest head, odd page size
+    dict(seq_lens=[50, 200], Hq=6, Hkv=3, D=80, P=16),              # 5 lanes of 8 per key
+])
+def test_attention_decode(ops, dtype, splits, case):
+    _attention_case(ops, dtype, q_lens=[1] * len(case["seq_lens"]), kernel="decode", splits=splits,
+                    **case)
+
+
+@pytest.mark.parametrize("dtype", DT, ids=IDS)
+def test_attention_decode_window(ops, dtype):
+    _attention_case(ops, dtype, seq_lens=[90, 40, 7], q_lens=[1, 1, 1], Hq=4, Hkv=2, D=32, P=8,
+                    window=20, kernel="decode", splits=2)
+
+
+@pytest.mark.parametrize("case", [
+    dict(seq_lens=[40], q_lens=[40], Hq=4, Hkv=4, D=64, P=16),
+    dict(seq_lens=[200, 64, 33], q_lens=[130, 2, 33], Hq=6, Hkv=1, D=128, P=8),
+    dict(seq_lens=[150], q_lens=[70], Hq=2, Hkv=1, D=32, P=5),
+    dict(seq_lens=[129, 300], q_lens=[129, 65], Hq=4, Hkv=2, D=96, P=16),
+    dict(seq_lens=[1, 2, 64, 65], q_lens=[1, 2, 64, 65], Hq=2, Hkv=2, D=64, P=4),
+])
+def test_attention_prefill_mfma(ops, case):
+    _attention_case(ops, torch.bfloat16, kernel="mfma", **case)
+
+
+def test_attention_prefill_mfma_window(ops):
+    _attention_case(ops, torch.bfloat16, seq_lens=[300, 90], q_lens=[150, 25], Hq=4, Hkv=2, D=64,
+                    P=8, window=70, kernel="mfma")
+
+
+@pytest.mark.parametrize("kernel", ["decode", "mfma"])
+def test_attention_far_key_stands_out_fast_kernels(ops, kernel):
+    def boost(q, dk, kc, bt):
+        direction = torch.ones(64) * 2.0
+        q[-1, :, :] = direction.to(q.dtype)
+        page = int(bt[0, 0])
+        kc[page, :, 3] = direction.to(kc.dtype)
+        dk[0][3] = direction
+    ql = 1 if kernel == "decode" else 2
+    _attention_case(ops, torch.bfloat16, seq_lens=[700], q_lens=[ql], Hq=2, Hkv=1, D=64, P=16,
+                    boost=boost, kernel=kernel, splits=4)
 
 
 @pytest.mark.parametrize("dtype", DT, ids=IDS)
