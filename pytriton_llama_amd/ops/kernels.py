@@ -176,6 +176,40 @@ def gemm_nt(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
     return y
 
 
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_skinny_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the weight-streaming matrix-core kernel takes this product."""
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
+            and 0 < x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0 and x.stride(1) == 1
+            and (x.shape[0] == 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0
+            and w.is_contiguous() and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y = x @ w.T for at most 64 rows of bfloat16 x, streaming w once
+    (see csrc/gemm.hip). Output bfloat16 or float32."""
+    _need_gpu(x, w)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelError(f"gemm_skinny: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
+    if not gemm_skinny_fits(x, w):
+        raise KernelError("gemm_skinny: needs bfloat16, at most 64 rows, K a multiple of 8 and "
+                          "16-byte aligned rows")
+    M, K = x.shape
+    N = w.shape[0]
+    out_dtype = out_dtype or torch.bfloat16
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError("gemm_skinny: output is bfloat16 or float32")
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    ldx = x.stride(0) if M > 1 else max(K, 8)
+    lib = library.load("gemm")
+    _check(lib.ptl_gemm_skinny_bf16(_ptr(y), _ptr(x), _ptr(w), M, N, K, ctypes.c_long(ldx),
+                                    ctypes.c_long(N), _F32 if out_dtype == torch.float32 else _BF16,
+                                    _stream()), "gemm_skinny")
+    return y
+
+
 def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                       block_table: torch.Tensor, work_seq: torch.Tensor, work_qoff: torch.Tensor,

@@ -24,6 +24,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
         return ops.gemm_nt(x, w, torch.float32)
+    if ops.gemm_skinny_fits(x, w):
+        return ops.gemm_skinny(x, w, out_dtype)
     if out_dtype == torch.float32:
         return ops.gemm_nt(x, w, torch.float32)
     return torch.nn.functional.linear(x, w)

@@ -81,6 +81,30 @@ def test_gemm_nt(ops, dtype, mnk):
                                **tol(dtype))
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["to_bf16", "to_fp32"])
+@pytest.mark.parametrize("mnk", [(1, 300, 72), (7, 65, 136), (16, 3072, 2048), (17, 100, 200),
+                                 (33, 16, 8192), (64, 1000, 64), (8, 2048, 8192), (5, 130, 2056)])
+def test_gemm_skinny(ops, out_dtype, mnk):
+    M, N, K = mnk
+    torch.manual_seed(7)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    want = (x.double() @ w.double().T).float()
+    y = ops.gemm_skinny(x, w, out_dtype)
+    assert y.dtype == out_dtype
+    t = dict(atol=1e-4, rtol=1e-4) if out_dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(y.float(), want, **t)
+    # rows of x as a slice of a wider buffer
+    wide = torch.randn(M, K + 24, device="cuda").to(torch.bfloat16)
+    xs = wide[:, 8:8 + K]
+    torch.testing.assert_close(ops.gemm_skinny(xs, w, out_dtype).float(),
+                               (xs.double() @ w.double().T).float(), **t)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(torch.zeros(65, K, device="cuda", dtype=torch.bfloat16), w)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(x[:, :K - 4], w[:, :K - 4].contiguous())
+
+
 def _rope_reference(x, positions, inv_freq):
     cos, sin = plain_llama.rope_cos_sin(inv_freq, positions)
     return plain_llama.apply_rope(x, cos, sin)
