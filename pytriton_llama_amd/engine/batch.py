@@ -78,10 +78,9 @@ def order_entries(entries: Sequence[StepEntry]) -> List[int]:
            [i for i in idx if len(entries[i].tokens) != 1]
 
 
-def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Optional[int] = None):
-    """Take pages for every entry (all or nothing) and lay the batch out.
-    Returns (StepContext, order) where ``order`` is the permutation applied to
-    the entries; logit rows are listed in the caller's order of entries."""
+def take_pages(entries: Sequence[StepEntry], manager, vocab_size: Optional[int] = None) -> List[int]:
+    """Check the entries and take the pages for all of them, or for none.
+    Returns the position of every entry's first token."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     seen = set()
@@ -100,7 +99,6 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
                 if not 0 <= t < vocab_size:
                     raise ValueError(f"request {e.request!r}: token id {t} outside the "
                                      f"vocabulary of {vocab_size}")
-    # pages: check the whole step before taking anything
     need = [0] * len(manager.paged)
     for e in entries:
         for g, n in enumerate(manager.pages_needed(e.request, len(e.tokens))):
@@ -110,6 +108,14 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
             from ..cache.manager import OutOfPages
             raise OutOfPages(f"the step needs {n} pages of group {g}, "
                              f"{manager.paged[g].pool.num_free} are free")
+    return [manager.append(e.request, len(e.tokens)) for e in entries]
+
+
+def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Optional[int] = None):
+    """Take pages for every entry (all or nothing) and lay the batch out.
+    Returns (StepContext, order) where ``order`` is the permutation applied to
+    the entries; logit rows are listed in the caller's order of entries."""
+    starts = take_pages(entries, manager, vocab_size)
 
     order = order_entries(entries)
     token_ids: List[int] = []
@@ -122,7 +128,7 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
     for i in order:
         e = entries[i]
         n = len(e.tokens)
-        start = manager.append(e.request, n)
+        start = starts[i]
         row_of_entry[i] = q_start[-1]
         token_ids.extend(int(t) for t in e.tokens)
         positions.extend(range(start, start + n))

@@ -57,7 +57,8 @@ class Engine:
             self.model = build_model(model)
             load_random_weights(self.model, random_seed or 0, ec.dtype, ec.device, norm_std, weight_std)
         num_pages = ec.num_pages if ec.num_pages is not None else pages_from_memory(self.model, ec)
-        self.runner = ModelRunner(self.model, ec.page_size, num_pages, ec.max_num_seqs)
+        self.runner = ModelRunner(self.model, ec.page_size, num_pages, ec.max_num_seqs,
+                                  ec.max_model_len, ec.use_graphs)
         eos = getattr(self.model.config, "eos_token_ids", ())
         self.scheduler = Scheduler(self.runner.manager, ec.max_num_seqs, ec.max_num_batched_tokens,
                                    ec.prefill_chunk, ec.max_model_len, eos)

@@ -20,7 +20,8 @@ class ModelRunner:
     is ModelExecutor.forward with prefill_alloc_kv_cache / decode_alloc_kv_cache
     around it (lite_llama/executor/model_executor.py:261-320)."""
 
-    def __init__(self, model, page_size: int, num_pages, max_num_seqs: int):
+    def __init__(self, model, page_size: int, num_pages, max_num_seqs: int,
+                 max_model_len: Optional[int] = None, use_graphs: bool = False):
         if model.dtype is None:
             raise RuntimeError("load the model's weights before making a runner")
         self.model = model
@@ -29,6 +30,11 @@ class ModelRunner:
             ops.library.require(model.kernel_libraries())
         self.manager = CacheManager(model.cache_layers, page_size, num_pages, max_num_seqs)
         self.storage = CacheStorage(self.manager, model.dtype, self.device)
+        # decode-only steps replay a HIP graph when the longest request is known
+        self.graphs = None
+        if use_graphs and max_model_len and self.device.type == "cuda" and not self.manager.states:
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(model, self.manager, self.storage, max_model_len, self.device)
 
     def admit(self, request: Hashable) -> None:
         slot = self.manager.admit(request)
@@ -41,8 +47,11 @@ class ModelRunner:
         for e in entries:
             if not self.manager.is_live(e.request):
                 self.admit(e.request)
-        ctx, _ = build_context(entries, self.manager, self.device, self.model.vocab_size)
-        logits = self.model.forward(ctx, self.storage)
+        if self.graphs is not None and self.graphs.fits(entries):
+            logits = self.graphs.step(entries)
+        else:
+            ctx, _ = build_context(entries, self.manager, self.device, self.model.vocab_size)
+            logits = self.model.forward(ctx, self.storage)
         for e in entries:
             self.manager.release_behind_window(e.request)
         return logits

@@ -119,3 +119,52 @@ def test_command_line(folder_a):
         capture_output=True, text=True, timeout=110)
     assert out.returncode == 0, out.stderr[-2000:]
     assert [int(x) for x in out.stdout.split()] == want
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_decode_graphs_match_eager_steps(folder_b, dtype):
+    """Decode-only steps replayed as HIP graphs give the logits of the same
+    steps launched kernel by kernel: every replay is checked, with eager work
+    (prompt portions of a newcomer, a request ending, another batch size) and
+    synchronisations between the replays."""
+    from pytriton_llama_amd.config import build_model, read_config_json
+    from pytriton_llama_amd.engine.batch import StepEntry
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_weights
+    folder, page = folder_b
+    model = build_model(read_config_json(folder))
+    load_weights(model, folder, dtype, "cuda:0")
+    eager = ModelRunner(model, page, 40, 6)
+    graphed = ModelRunner(model, page, 40, 6, max_model_len=200, use_graphs=True)
+    assert graphed.graphs is not None and eager.graphs is None
+    g = torch.Generator().manual_seed(12)
+    toks = {r: torch.randint(0, 384, (160,), generator=g).tolist() for r in "abcd"}
+    fed = {r: 0 for r in toks}
+
+    def both(spec):
+        entries = []
+        for r, n in spec:
+            entries.append(StepEntry(r, toks[r][fed[r]:fed[r] + n], [n - 1]))
+            fed[r] += n
+        le = eager.step(entries).float().cpu()
+        lg = graphed.step(entries).float().cpu()
+        scale = float(le.abs().max())
+        assert float((le - lg).abs().max()) / scale < (1e-5 if dtype == torch.float32 else 2e-2)
+
+    both([("a", 37), ("b", 5), ("c", 70)])                # prompts: eager in both runners
+    replays = 0
+    for i in range(40):
+        both([("a", 1), ("b", 1), ("c", 1)])              # bucket of 4, three live rows
+        replays += 1
+        if i == 10:
+            both([("d", 33), ("a", 1)])                   # mixed step between replays: eager
+        if i > 10 and i % 2:
+            both([("d", 1)])                              # another bucket
+        if i == 25:
+            for r in (eager, graphed):
+                r.end("b")
+            toks["b"] = toks["b"][::-1]
+            fed["b"] = 0
+            both([("b", 9)])                              # a new request in the freed pages
+    assert graphed.graphs.buckets[4].graph is not None and graphed.graphs.buckets[1].graph is not None
+    assert replays == 40
