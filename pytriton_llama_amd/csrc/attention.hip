@@ -369,24 +369,34 @@ attn_decode_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ q
 }
 
 template <typename T>
-__global__ void attn_decode_merge_kernel(T* __restrict__ out, long out_stride,
-                                         const int32_t* __restrict__ q_start,
-                                         const float* __restrict__ part_acc,
-                                         const float* __restrict__ part_ml,
-                                         int Hq, int D, int num_splits) {
-  const int seq = blockIdx.x, head = blockIdx.y;
+__global__ void __launch_bounds__(64)
+attn_decode_merge_kernel(T* __restrict__ out, long out_stride, const int32_t* __restrict__ q_start,
+                         const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                         int Hq, int D, int num_splits) {
+  // one wave per (sequence, head): lanes take the splits' (max, denominator) side by side,
+  // then the head dimension, with the splits' weights in LDS
+  __shared__ float wgt[1024];
+  const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const size_t base = ((size_t)seq * Hq + head) * num_splits;
   float mn = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) mn = fmaxf(mn, part_ml[(base + s) * 2]);
+  for (int s = lane; s < num_splits; s += 64) mn = fmaxf(mn, part_ml[(base + s) * 2]);
+  mn = wave_max(mn);
   const float ms = mn == -INFINITY ? 0.f : mn;
   float ll = 0.f;
-  for (int s = 0; s < num_splits; ++s) ll += part_ml[(base + s) * 2 + 1] * expf(part_ml[(base + s) * 2] - ms);
+  for (int s = lane; s < num_splits; s += 64) {
+    const float w = expf(part_ml[(base + s) * 2] - ms);
+    if (s < 1024) wgt[s] = w;
+    ll += part_ml[(base + s) * 2 + 1] * w;
+  }
+  ll = wave_sum(ll);
+  __syncthreads();
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;
   const int row = q_start[seq];
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+  for (int d = lane; d < D; d += 64) {
     float a = 0.f;
-    for (int s = 0; s < num_splits; ++s)
-      a += part_acc[(base + s) * D + d] * expf(part_ml[(base + s) * 2] - ms);
+    const float* pa = part_acc + base * D + d;
+#pragma unroll 8
+    for (int s = 0; s < num_splits; ++s) a = fmaf(pa[(size_t)s * D], wgt[s], a);
     out[(size_t)row * out_stride + (size_t)head * D + d] = from_float<T>(a * inv);
   }
 }
@@ -427,7 +437,7 @@ extern "C" int ptl_attention_decode(void* out, long out_stride, const void* q, l
                                     hipStream_t stream) {
   if (n_seq <= 0) return PTL_OK;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D <= 0 || D % 16 || D > 256 || page_size <= 0 ||
-      num_splits < 1 || num_splits > 65535 || (num_splits > 1 && (!part_acc || !part_ml)))
+      num_splits < 1 || num_splits > 1024 || (num_splits > 1 && (!part_acc || !part_ml)))
     return PTL_ERR_ARG;
   const int chunks = D / 16;
   int lpk = 1;
@@ -672,6 +682,248 @@ extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void
 #define GO(N) launch_prefill_mfma<N>(out, out_stride, q, q_stride, k_cache, v_cache, q_start,      \
                                      ctx_len, block_table, bt_stride, work_seq, work_qoff, n_work, \
                                      Hq, Hkv, page_size, window, scale, stream)
+  switch (D / 32) {
+    case 1: return GO(1);
+    case 2: return GO(2);
+    case 3: return GO(3);
+    default: return GO(4);
+  }
+#undef GO
+}
+
+// ===========================================================================
+// ptl_attention_decode_mfma: the bfloat16 decode case on the matrix cores.
+//
+// Same grid and split scheme as ptl_attention_decode, but a wave takes 16 keys
+// per turn and all query heads of a kv head at once (up to 16 of them are the N
+// side of the MFMA tiles, so grouped heads cost nothing extra):
+//   S^T[key, head] = K[key, :] . Q[head, :]         v_mfma_f32_16x16x32_bf16,
+//                                                   A = 16-byte loads of key rows
+//   O^T[d, head]  += V^T[d, key] . P^T[key, head]   v_mfma_f32_16x16x16_bf16,
+//                                                   B = P^T as it leaves the
+//                                                   first product, A = values
+//                                                   gathered by (d, key)
+// The softmax state of a head (running max, denominator) lives in the lanes of
+// that head's column; the four waves and the splits are merged at the end as
+// in ptl_attention_decode. Needs D % 32 == 0, D <= 128, Hq/Hkv <= 16.
+// ===========================================================================
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+template <int NDT>
+__global__ void __launch_bounds__(256)
+attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
+                        long q_stride, const bf16_t* __restrict__ k_cache,
+                        const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ q_start,
+                        const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ block_table,
+                        int bt_stride, float* __restrict__ part_acc, float* __restrict__ part_ml,
+                        int Hq, int Hkv, int page_size, int window, float scale_log2, int num_splits) {
+  constexpr int D = 32 * NDT;
+  constexpr int NT = 2 * NDT;             // 16-wide tiles of the head dimension
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ln = lane & 15, lg = lane >> 4;
+  const int seq = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int G = Hq / Hkv;
+  const int head0 = kvh * G;
+  const int row = q_start[seq];
+  const int ctx = ctx_len[seq];
+  const int k_lo = window > 0 ? max(0, ctx - window) : 0;
+  const int span = ctx - k_lo;
+  constexpr int UNR = NDT <= 2 ? 4 : 2;   // 16-key tiles a wave loads ahead
+  constexpr int TILE = 64 * UNR;          // keys per turn of the workgroup
+  const int per_split = ((span + num_splits - 1) / num_splits + TILE - 1) / TILE * TILE;
+  const int k_begin = k_lo + split * per_split;
+  const int k_end = min(ctx, k_begin + per_split);
+  const int32_t* bt = block_table + (size_t)seq * bt_stride;
+  const size_t head_pages = (size_t)Hkv * page_size * D;     // elements per page
+  const size_t kv_off = (size_t)kvh * page_size * D;
+
+  Frag8 qf[NDT];
+#pragma unroll
+  for (int kk = 0; kk < NDT; ++kk) {
+    qf[kk].u = make_uint4(0, 0, 0, 0);
+    if (ln < G)
+      qf[kk].u = *reinterpret_cast<const uint4*>(q + (size_t)row * q_stride +
+                                                 (size_t)(head0 + ln) * D + 32 * kk + 8 * lg);
+  }
+  f32x4_t o[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) o[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_part = 0.f;
+
+  // values go through LDS: each wave copies its tiles row by row (coalesced 16-byte
+  // loads) into a region of its own and reads them back by (d, key) for the second product
+  constexpr int VS = D + 4;               // row stride in elements: rows 4 apart fall 8 banks apart
+  constexpr int CPR = D / 8;              // 16-byte chunks per row
+  constexpr int VCH = 16 * CPR / 64;      // chunks of a tile per lane
+  extern __shared__ float lds[];
+  bf16_t* vl = reinterpret_cast<bf16_t*>(lds) + (size_t)wave * UNR * 16 * VS;
+  const int turns = (k_end - k_begin + TILE - 1) / TILE;
+  for (int turn = 0; turn < turns; ++turn) {
+    const int kc = k_begin + turn * TILE + 16 * UNR * wave;
+    Frag8 kf[UNR][NDT];
+    uint4 vg[UNR][VCH];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int kb = kc + 16 * u;
+      {
+        const int kp = kb + ln;                   // row ln of the key tile (first product)
+        const bool ok = kp < k_end;
+        const bf16_t* kr = k_cache;
+        if (ok) {
+          const int page = bt[kp / page_size];
+          kr = k_cache + (size_t)page * head_pages + kv_off + (size_t)(kp % page_size) * D + 8 * lg;
+        }
+#pragma unroll
+        for (int kk = 0; kk < NDT; ++kk)
+          kf[u][kk].u = ok ? *reinterpret_cast<const uint4*>(kr + 32 * kk) : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < VCH; ++i) {
+        const int c = lane + 64 * i;
+        const int kp = kb + c / CPR;
+        vg[u][i] = make_uint4(0, 0, 0, 0);
+        if (kp < k_end) {
+          const int page = bt[kp / page_size];
+          vg[u][i] = *reinterpret_cast<const uint4*>(
+              v_cache + (size_t)page * head_pages + kv_off + (size_t)(kp % page_size) * D + (c % CPR) * 8);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+#pragma unroll
+      for (int i = 0; i < VCH; ++i) {
+        const int c = lane + 64 * i;
+        uint2* dst = reinterpret_cast<uint2*>(vl + (size_t)(u * 16 + c / CPR) * VS + (c % CPR) * 8);
+        dst[0] = make_uint2(vg[u][i].x, vg[u][i].y);
+        dst[1] = make_uint2(vg[u][i].z, vg[u][i].w);
+      }
+    __syncthreads();
+    s16x4_t vf[UNR][NT];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          vf[u][t][j] = (short)vl[(size_t)(u * 16 + 4 * lg + j) * VS + 16 * t + ln];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int kb = kc + 16 * u;
+      if (kb >= k_end) break;                     // wave-uniform
+      f32x4_t st = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NDT; ++kk)
+        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][kk].v, qf[kk].v, st, 0, 0, 0);
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float s = st[i] * scale_log2;
+        s = (kb + 4 * lg + i < k_end) ? s : -INFINITY;
+        st[i] = s;
+        tmax = fmaxf(tmax, s);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run, tmax);      // finite: key kb is in range
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      l_part *= alpha;
+      s16x4_t pb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __builtin_amdgcn_exp2f(st[i] - m_new);
+        l_part += p;
+        pb[i] = (short)float_to_bf16(p);
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        o[t][0] *= alpha; o[t][1] *= alpha; o[t][2] *= alpha; o[t][3] *= alpha;
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[u][t], pb, o[t], 0, 0, 0);
+      }
+    }
+  }
+
+  float l = l_part + __shfl_xor(l_part, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+
+  // merge the four waves: [wave][head][D] accumulators, [wave][head][2] (max, denominator);
+  // the region takes the place of the value tiles, which every wave has left by now
+  __syncthreads();
+  float* w_acc = lds;
+  float* w_ml = lds + 4 * 16 * D;
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w_acc[((wave * 16 + ln) * D) + 16 * t + 4 * lg + i] = o[t][i];
+  if (lg == 0) { w_ml[(wave * 16 + ln) * 2] = m_run; w_ml[(wave * 16 + ln) * 2 + 1] = l; }
+  __syncthreads();
+  for (int i = tid; i < G * D; i += 256) {
+    const int h = i / D, d = i - h * D;
+    float mn = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mn = fmaxf(mn, w_ml[(w * 16 + h) * 2]);
+    const float ms = mn == -INFINITY ? 0.f : mn;
+    float ll = 0.f, a = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = __builtin_amdgcn_exp2f(w_ml[(w * 16 + h) * 2] - ms);
+      ll += w_ml[(w * 16 + h) * 2 + 1] * f;
+      a += w_acc[(w * 16 + h) * D + d] * f;
+    }
+    const int head = head0 + h;
+    if (num_splits == 1) {
+      out[(size_t)row * out_stride + (size_t)head * D + d] = float_to_bf16(ll > 0.f ? a / ll : 0.f);
+    } else {
+      const size_t pi = ((size_t)seq * Hq + head) * num_splits + split;
+      part_acc[pi * D + d] = a;
+      // the merge kernel works with natural exponents
+      if (d == 0) { part_ml[pi * 2] = mn * 0.6931471805599453f; part_ml[pi * 2 + 1] = ll; }
+    }
+  }
+}
+
+template <int NDT>
+static int launch_decode_mfma(void* out, long out_stride, const void* q, long q_stride,
+                              const void* k_cache, const void* v_cache, const int32_t* q_start,
+                              const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
+                              float* part_acc, float* part_ml, int n_seq, int Hq, int Hkv,
+                              int page_size, int window, float scale, int num_splits,
+                              hipStream_t stream) {
+  constexpr int D = 32 * NDT;
+  constexpr int UNR = NDT <= 2 ? 4 : 2;
+  dim3 grid(n_seq, Hkv, num_splits);
+  const size_t lds_merge = (size_t)(4 * 16 * D + 4 * 16 * 2) * sizeof(float);
+  const size_t lds_values = (size_t)4 * UNR * 16 * (D + 4) * sizeof(bf16_t);
+  const size_t lds = lds_merge > lds_values ? lds_merge : lds_values;
+  attn_decode_mfma_kernel<NDT><<<grid, 256, lds, stream>>>(
+      (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
+      (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv,
+      page_size, window, scale * 1.4426950408889634f, num_splits);
+  if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
+  if (num_splits > 1) {
+    dim3 mgrid(n_seq, Hq);
+    attn_decode_merge_kernel<bf16_t><<<mgrid, 64, 0, stream>>>((bf16_t*)out, out_stride, q_start,
+                                                              part_acc, part_ml, Hq, D, num_splits);
+  }
+  return ptl_launch_status();
+}
+
+extern "C" int ptl_attention_decode_mfma(void* out, long out_stride, const void* q, long q_stride,
+                                         const void* k_cache, const void* v_cache,
+                                         const int32_t* q_start, const int32_t* ctx_len,
+                                         const int32_t* block_table, int bt_stride, float* part_acc,
+                                         float* part_ml, int n_seq, int Hq, int Hkv, int D,
+                                         int page_size, int window, float scale, int num_splits,
+                                         hipStream_t stream) {
+  if (n_seq <= 0) return PTL_OK;
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 16 || D <= 0 || D % 32 || D > 128 ||
+      page_size <= 0 || q_stride % 8 || num_splits < 1 || num_splits > 1024 ||
+      (num_splits > 1 && (!part_acc || !part_ml)))
+    return PTL_ERR_ARG;
+#define GO(N) launch_decode_mfma<N>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len, \
+                                    block_table, bt_stride, part_acc, part_ml, n_seq, Hq, Hkv,      \
+                                    page_size, window, scale, num_splits, stream)
   switch (D / 32) {
     case 1: return GO(1);
     case 2: return GO(2);

@@ -88,30 +88,37 @@ class PagedAttention(Part):
         return linear(out.view(T, Hq * D), self.o)
 
     # ---- which kernel takes which sequences --------------------------------------
-    def decode_splits(self, ctx, n_dec: int) -> int:
+    def decode_splits(self, ctx, n_dec: int, matrix_cores: bool) -> int:
         """How many workgroups share one sequence's keys: enough to fill the 256
         CUs a few times over, never finer than one turn of a workgroup."""
         if self.force_decode_splits:
             return self.force_decode_splits
         D = self.head_dim
-        lpk = 1
-        while lpk * 16 < D:
-            lpk <<= 1
-        tile = 256 // lpk
-        groups = self.num_kv_heads * (-(-(self.num_heads // self.num_kv_heads) // 4))
+        G = self.num_heads // self.num_kv_heads
+        if matrix_cores:
+            turn = 256 if D <= 64 else 128          # keys a workgroup takes per turn
+            groups = self.num_kv_heads
+        else:
+            lpk = 1
+            while lpk * 16 < D:
+                lpk <<= 1
+            turn = 2 * (256 // lpk)
+            groups = self.num_kv_heads * (-(-G // 4))
         span = max(ctx.ctx_lens[:n_dec])
         if self.window:
             span = min(span, self.window)
-        want = -(-1024 // max(1, n_dec * groups))
-        return max(1, min(want, -(-span // tile), 64))
+        want = -(-768 // max(1, n_dec * groups))
+        return max(1, min(want, -(-span // turn), 64))
 
     def attend(self, out, q, cache, ctx, group) -> None:
         D, window = self.head_dim, self.window or 0
         n_dec = ctx.num_decode_seqs if D % 16 == 0 else 0
         if n_dec:
+            mfma = (ops.attention_decode_mfma_fits(q.dtype, self.num_heads, self.num_kv_heads, D)
+                    and q.stride(0) % 8 == 0)
             ops.attention_decode(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
                                  group.block_table, n_dec, self.scale, window,
-                                 self.decode_splits(ctx, n_dec))
+                                 self.decode_splits(ctx, n_dec, mfma), matrix_cores=mfma)
         if n_dec == ctx.num_seqs:
             return
         if q.dtype == torch.bfloat16 and D % 32 == 0 and D <= 128:

@@ -206,7 +206,8 @@ def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=
     else:
         assert all(ql == 1 for ql in q_lens)
         ops.attention_decode(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
-                             bt.to(dev), len(q_lens), scale, window, splits)
+                             bt.to(dev), len(q_lens), scale, window, splits,
+                             matrix_cores=(kernel == "decode_mfma"))
     # plain: full causal attention over the sequence, rows of the portion kept
     for i, (s, ql) in enumerate(zip(seq_lens, q_lens)):
         full_q = torch.zeros(s, Hq, D)
@@ -244,6 +245,23 @@ def test_attention_decode(ops, dtype, splits, case):
                     **case)
 
 
+@pytest.mark.parametrize("splits", [1, 2, 5])
+@pytest.mark.parametrize("case", [
+    dict(seq_lens=[300, 64, 65, 1], Hq=4, Hkv=4, D=64, P=16),
+    dict(seq_lens=[100, 257], Hq=32, Hkv=2, D=32, P=8),             # 16 heads a kv head
+    dict(seq_lens=[90, 33, 700], Hq=3, Hkv=1, D=128, P=16),
+    dict(seq_lens=[70, 130], Hq=8, Hkv=2, D=96, P=5),               # odd page size
+])
+def test_attention_decode_mfma(ops, splits, case):
+    _attention_case(ops, torch.bfloat16, q_lens=[1] * len(case["seq_lens"]), kernel="decode_mfma",
+                    splits=splits, **case)
+
+
+def test_attention_decode_mfma_window(ops):
+    _attention_case(ops, torch.bfloat16, seq_lens=[90, 40, 7], q_lens=[1, 1, 1], Hq=4, Hkv=2, D=32,
+                    P=8, window=20, kernel="decode_mfma", splits=2)
+
+
 @pytest.mark.parametrize("dtype", DT, ids=IDS)
 def test_attention_decode_window(ops, dtype):
     _attention_case(ops, dtype, seq_lens=[90, 40, 7], q_lens=[1, 1, 1], Hq=4, Hkv=2, D=32, P=8,
@@ -266,7 +284,7 @@ def test_attention_prefill_mfma_window(ops):
                     P=8, window=70, kernel="mfma")
 
 
-@pytest.mark.parametrize("kernel", ["decode", "mfma"])
+@pytest.mark.parametrize("kernel", ["decode", "decode_mfma", "mfma"])
 def test_attention_far_key_stands_out_fast_kernels(ops, kernel):
     def boost(q, dk, kc, bt):
         direction = torch.ones(64) * 2.0
@@ -274,7 +292,7 @@ def test_attention_far_key_stands_out_fast_kernels(ops, kernel):
         page = int(bt[0, 0])
         kc[page, :, 3] = direction.to(kc.dtype)
         dk[0][3] = direction
-    ql = 1 if kernel == "decode" else 2
+    ql = 2 if kernel == "mfma" else 1
     _attention_case(ops, torch.bfloat16, seq_lens=[700], q_lens=[ql], Hq=2, Hkv=1, D=64, P=16,
                     boost=boost, kernel=kernel, splits=4)
 
