@@ -19,40 +19,62 @@
 #include "common.h"
 #include <math.h>
 
-__global__ void argmax_kernel(int32_t* __restrict__ out, const float* __restrict__ logits,
-                              int V, long stride) {
-  __shared__ float sv[16];
-  __shared__ int si[16];
-  const float* row = logits + (size_t)blockIdx.x * stride;
+// Two passes so that a row of vocabulary size is read by many workgroups: every
+// chunk leaves its best (value, index), then one wave per row picks among them.
+#define ARGMAX_CHUNK 4096
+
+__device__ __forceinline__ void argmax_pick(float& best, int& bi, float v, int i) {
+  if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+}
+
+__global__ void __launch_bounds__(256)
+argmax_partial_kernel(float* __restrict__ pv, int32_t* __restrict__ pi,
+                      const float* __restrict__ logits, int V, long stride, int chunks) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  const float* row = logits + (size_t)blockIdx.y * stride;
+  const int lo = blockIdx.x * ARGMAX_CHUNK, hi = min(V, lo + ARGMAX_CHUNK);
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+  for (int i = lo + threadIdx.x; i < hi; i += 256) {
     float v = row[i];
     if (v != v) v = -INFINITY;
-    if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+    argmax_pick(best, bi, v, i);
   }
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const float ov = __shfl_xor(best, o, 64);
-    const int oi = __shfl_xor(bi, o, 64);
-    if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-  }
+  for (int o = 32; o > 0; o >>= 1) argmax_pick(best, bi, __shfl_xor(best, o, 64), __shfl_xor(bi, o, 64));
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (lane == 0) { sv[wave] = best; si[wave] = bi; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int nw = blockDim.x >> 6;
-    for (int i = 1; i < nw; ++i)
-      if (sv[i] > best || (sv[i] == best && si[i] < bi)) { best = sv[i]; bi = si[i]; }
-    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    for (int i = 1; i < 4; ++i) argmax_pick(best, bi, sv[i], si[i]);
+    pv[(size_t)blockIdx.y * chunks + blockIdx.x] = best;
+    pi[(size_t)blockIdx.y * chunks + blockIdx.x] = bi;
   }
 }
 
+__global__ void __launch_bounds__(64)
+argmax_final_kernel(int32_t* __restrict__ out, const float* __restrict__ pv,
+                    const int32_t* __restrict__ pi, int chunks) {
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < chunks; i += 64)
+    argmax_pick(best, bi, pv[(size_t)blockIdx.x * chunks + i], pi[(size_t)blockIdx.x * chunks + i]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) argmax_pick(best, bi, __shfl_xor(best, o, 64), __shfl_xor(bi, o, 64));
+  if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
+// workspace: float [R, chunks] and int32 [R, chunks], chunks = ceil(V / 4096)
 extern "C" int ptl_argmax(int32_t* out, const float* logits, int R, int V, long stride,
-                          hipStream_t stream) {
+                          float* ws_val, int32_t* ws_idx, hipStream_t stream) {
   if (R <= 0) return PTL_OK;
-  if (V <= 0 || stride < V) return PTL_ERR_ARG;
-  argmax_kernel<<<R, 1024, 0, stream>>>(out, logits, V, stride);
+  if (V <= 0 || stride < V || !ws_val || !ws_idx || R > 65535) return PTL_ERR_ARG;
+  const int chunks = (V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+  dim3 grid(chunks, R);
+  argmax_partial_kernel<<<grid, 256, 0, stream>>>(ws_val, ws_idx, logits, V, stride, chunks);
+  if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
+  argmax_final_kernel<<<R, 64, 0, stream>>>(out, ws_val, ws_idx, chunks);
   return ptl_launch_status();
 }
 

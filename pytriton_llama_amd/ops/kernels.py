@@ -351,9 +351,12 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
         raise KernelError("argmax: logits must be float32 [R, V] with dense rows")
     R, V = logits.shape
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    chunks = -(-V // 4096)
+    ws_val = torch.empty((R, chunks), dtype=torch.float32, device=logits.device)
+    ws_idx = torch.empty((R, chunks), dtype=torch.int32, device=logits.device)
     lib = library.load("sampling")
-    _check(lib.ptl_argmax(_ptr(out), _ptr(logits), R, V, ctypes.c_long(logits.stride(0)), _stream()),
-           "argmax")
+    _check(lib.ptl_argmax(_ptr(out), _ptr(logits), R, V, ctypes.c_long(logits.stride(0)),
+                          _ptr(ws_val), _ptr(ws_idx), _stream()), "argmax")
     return out
 
 

@@ -16,6 +16,8 @@ import torch
 from .. import ops
 
 LINEAR_LIBRARIES = ("gemm",)
+SKINNY_ROWS = 8          # rows up to which the skinny kernel takes a bfloat16 product
+SKINNY_ROWS_F32 = 16     # ... when float32 output is wanted (the head)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -24,8 +26,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
         return ops.gemm_nt(x, w, torch.float32)
-    if ops.gemm_skinny_fits(x, w):
+    M = x.shape[0]
+    to_f32 = out_dtype == torch.float32
+    # measured on MI355X at the 1B shapes: the weight-streaming kernel is level with the
+    # library up to 8 rows (and ahead for the vocabulary-sized head); beyond that the library
+    if ops.gemm_skinny_fits(x, w) and (M <= SKINNY_ROWS or (to_f32 and M <= SKINNY_ROWS_F32)):
         return ops.gemm_skinny(x, w, out_dtype)
-    if out_dtype == torch.float32:
+    if to_f32:
+        if x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
+            return torch.mm(x, w.t(), out_dtype=torch.float32)
         return ops.gemm_nt(x, w, torch.float32)
     return torch.nn.functional.linear(x, w)

@@ -337,10 +337,12 @@ def test_attention_page_placement_does_not_matter(ops):
     assert torch.equal(outs[0], outs[1])
 
 
-def test_argmax(ops):
+@pytest.mark.parametrize("V", [1003, 4096, 128256])
+def test_argmax(ops, V):
     torch.manual_seed(5)
-    logits = torch.randn(6, 1003, device="cuda")
-    logits[2, 7] = logits[2, 900] = 50.0       # a tie goes to the lowest id
+    logits = torch.randn(6, V, device="cuda")
+    logits[2, 7] = logits[2, V - 100] = 50.0       # a tie goes to the lowest id, across chunks too
+    logits[4, V - 1] = 60.0
     got = ops.argmax(logits).cpu()
     want = torch.argmax(logits.cpu(), dim=-1)
     want[2] = 7
