@@ -65,6 +65,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other batch sizes to report, '' for none")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--prefill-only", action="store_true", help="measure the prefill and stop (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
@@ -122,6 +123,10 @@ def main():
         prefill = {"value": round(S / best, 1), "tokens": S, "ms": round(best * 1e3, 3),
                    "frac": round(flops / best / PEAK_FLOPS[short], 4)}
         log(f"prefill {S} tokens: {best * 1e3:.2f} ms ({S / best:.0f} tok/s)")
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill}), flush=True)
+        return 0
 
     # ---- decode ---------------------------------------------------------------------
     def decode_rate(batch, steps, warmup):
