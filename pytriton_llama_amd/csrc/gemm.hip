@@ -141,8 +141,9 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
       const bool ok = kk + 8 * lg < ke;
       wf[u].u = ok ? *reinterpret_cast<const uint4*>(wp + kk) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        xf[t][u].u = ok ? *reinterpret_cast<const uint4*>(xp[t] + kk) : make_uint4(0, 0, 0, 0);
+      for (int t = 0; t < MT; ++t)   // columns past the last row of x are never stored: no load
+        xf[t][u].u = (ok && 16 * t + ln < M) ? *reinterpret_cast<const uint4*>(xp[t] + kk)
+                                             : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -182,8 +183,11 @@ static int launch_skinny(void* y, const void* x, const void* w, int M, int N, in
   const int blocks = (N + 15) / 16;
   // enough waves to keep every SIMD of 256 CUs busy a few times over, each with
   // at least 256 elements of K to stream
+  // (measured on MI355X: 4 waves a workgroup are best from N = 2048 to N = 128256 at
+  // K = 2048, 8 to 16 at K = 8192)
   int waves = 1;
   while (waves < 16 && (long)blocks * waves < 4096 && K / (waves * 2) >= 256) waves <<= 1;
+  if (waves < 4 && K >= 1024) waves = 4;
   int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * MT * 64 * 4 * sizeof(float) : 0;
   if (out_dtype == PTL_DTYPE_F32)

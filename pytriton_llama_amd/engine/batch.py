@@ -15,7 +15,8 @@ from typing import Hashable, List, Optional, Sequence
 import torch
 
 GENERIC_BLOCK_ROWS = 16   # query rows per work item of the vector-FMA attention kernel
-MFMA_BLOCK_ROWS = 64      # ... of the matrix-core prefill kernel
+MFMA_BLOCK_ROWS = 64      # ... of the matrix-core prefill kernel, for short portions
+MFMA_BIG_BLOCK_ROWS = 128  # ... and for long ones
 
 
 def work_items(q_lens, ctx_lens, first_seq: int, block_rows: int):
@@ -56,8 +57,8 @@ class StepContext:
     logit_rows: torch.Tensor       # int32 [R]: rows whose logits are wanted
     work: dict                     # name -> (sequence int32 [W], first query row int32 [W]):
                                    # "all16": 16-row blocks of every sequence; "multi16" /
-                                   # "multi64": 16- / 64-row blocks of the sequences after the
-                                   # leading single-token ones
+                                   # "multi64" / "multi128": 16- / 64- / 128-row blocks of the
+                                   # sequences after the leading single-token ones
     groups: List[GroupContext]
     num_tokens: int
     num_seqs: int
@@ -146,7 +147,8 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
         num_decode += 1
     work = {"all16": work_items(q_lens, ctx_len, 0, GENERIC_BLOCK_ROWS),
             "multi16": work_items(q_lens, ctx_len, num_decode, GENERIC_BLOCK_ROWS),
-            "multi64": work_items(q_lens, ctx_len, num_decode, MFMA_BLOCK_ROWS)}
+            "multi64": work_items(q_lens, ctx_len, num_decode, MFMA_BLOCK_ROWS),
+            "multi128": work_items(q_lens, ctx_len, num_decode, MFMA_BIG_BLOCK_ROWS)}
     tables = []
     for g, group in enumerate(manager.paged):
         rows = [group.tables[entries[i].request] for i in order]

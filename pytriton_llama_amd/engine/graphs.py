@@ -69,7 +69,8 @@ class _Bucket:
             token_ids=self.view("token_ids"), positions=self.view("positions"),
             q_start=self.view("q_start"), ctx_len=self.view("ctx_len"),
             state_slots=self.view("state_slots"), logit_rows=self.view("logit_rows"),
-            work={"all16": all16, "multi16": (empty, empty), "multi64": (empty, empty)},
+            work={"all16": all16, "multi16": (empty, empty), "multi64": (empty, empty),
+                  "multi128": (empty, empty)},
             groups=groups,
             num_tokens=B, num_seqs=B, num_logit_rows=B, logit_rows_are_identity=True,
             num_decode_seqs=B, q_lens=[1] * B, ctx_lens=[0] * B, max_q_len=1, max_ctx_len=0)

@@ -86,7 +86,7 @@ class Engine:
         plan = self.scheduler.schedule()
         entries, samplers = [], []
         for e in plan.entries:
-            toks = e.request.tokens[e.start:e.start + e.num_tokens]
+            toks = e.request.token_slice(e.start, e.num_tokens)
             entries.append(StepEntry(e.request.id, toks, [e.num_tokens - 1] if e.samples else []))
             if e.samples:
                 samplers.append(e.request)

@@ -29,7 +29,7 @@ class SamplingParams:
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
 
 
-@dataclass
+@dataclass(eq=False)          # a request is itself: compared and hashed by identity
 class Request:
     id: Hashable
     prompt: List[int]
@@ -43,6 +43,15 @@ class Request:
     @property
     def tokens(self) -> List[int]:
         return self.prompt + self.output
+
+    def token_slice(self, start: int, n: int) -> List[int]:
+        """tokens[start:start+n] without joining prompt and output."""
+        np_ = len(self.prompt)
+        if start + n <= np_:
+            return self.prompt[start:start + n]
+        if start >= np_:
+            return self.output[start - np_:start - np_ + n]
+        return self.prompt[start:] + self.output[:start + n - np_]
 
     @property
     def num_tokens(self) -> int:

@@ -117,13 +117,13 @@ class Scheduler:
         budget = self.max_num_batched_tokens
         # 1. decodes, in order of admission
         for req in list(self.running):
-            if req not in self.running or req.remaining != 1 or budget <= 0:
+            if req.status != RUNNING or req.remaining != 1 or budget <= 0:
                 continue
             if self._try_plan(req, 1, plan, reserve):
                 budget -= 1
         # 2. portions of prompts that are already running
         for req in list(self.running):
-            if req not in self.running or req.remaining <= 1 or budget <= 0:
+            if req.status != RUNNING or req.remaining <= 1 or budget <= 0:
                 continue
             n = min(req.remaining, self.prefill_chunk, budget)
             if self._try_plan(req, n, plan, reserve):

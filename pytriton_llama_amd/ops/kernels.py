@@ -319,9 +319,10 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
 def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                            v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                            block_table: torch.Tensor, work_seq: torch.Tensor,
-                           work_qoff: torch.Tensor, scale: float, window: int = 0) -> None:
+                           work_qoff: torch.Tensor, scale: float, window: int = 0,
+                           block_rows: int = 64) -> None:
     """bfloat16 attention of prompt portions on the matrix cores; the work list
-    names 64-row query blocks. Head sizes 32, 64, 96, 128."""
+    names query blocks of ``block_rows`` (64 or 128) rows. Head sizes 32, 64, 96, 128."""
     T, Hq, Hkv, D, page_size = _attention_common(out, q, k_cache, v_cache, q_start, ctx_len,
                                                  block_table, "attention_prefill_mfma")
     if q.dtype != torch.bfloat16:
@@ -333,6 +334,8 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
     _i32(work_qoff, "work_qoff")
     if work_seq.numel() != work_qoff.numel():
         raise KernelError("attention_prefill_mfma: inconsistent work list")
+    if block_rows not in (64, 128):
+        raise KernelError("attention_prefill_mfma: query blocks are 64 or 128 rows")
     if q.stride(0) % 8 or out.stride(0) % 4 or q.data_ptr() % 16 or out.data_ptr() % 8:
         raise KernelError("attention_prefill_mfma: q rows must be 16-byte aligned, out rows 8-byte")
     lib = library.load("attention")
@@ -340,7 +343,7 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
         _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
         _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
         int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), int(work_seq.numel()),
-        Hq, Hkv, D, page_size, int(window), ctypes.c_float(scale), _stream()),
+        int(block_rows), Hq, Hkv, D, page_size, int(window), ctypes.c_float(scale), _stream()),
         "attention_prefill_mfma")
 
 

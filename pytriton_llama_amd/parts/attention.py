@@ -122,9 +122,11 @@ class PagedAttention(Part):
         if n_dec == ctx.num_seqs:
             return
         if q.dtype == torch.bfloat16 and D % 32 == 0 and D <= 128:
-            ws, wo = ctx.work["multi64"]
+            # long portions in 128-row blocks (keys and values are staged half as often)
+            rows = 128 if ctx.max_q_len >= 256 else 64
+            ws, wo = ctx.work["multi128" if rows == 128 else "multi64"]
             ops.attention_prefill_mfma(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
-                                       group.block_table, ws, wo, self.scale, window)
+                                       group.block_table, ws, wo, self.scale, window, rows)
         else:
             ws, wo = ctx.work["multi16"] if n_dec else ctx.work["all16"]
             ops.attention_generic(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,

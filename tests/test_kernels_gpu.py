@@ -183,7 +183,7 @@ def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=
     q_start = [0]
     for ql in q_lens:
         q_start.append(q_start[-1] + ql)
-    rows = 64 if kernel == "mfma" else 16
+    rows = {"mfma": 64, "mfma128": 128}.get(kernel, 16)
     work_seq, work_qoff = [], []
     for s, ql in enumerate(q_lens):
         for off in range(0, ql, rows):
@@ -200,9 +200,9 @@ def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=
     if kernel == "generic":
         ops.attention_generic(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
                               bt.to(dev), i32(work_seq), i32(work_qoff), scale, window)
-    elif kernel == "mfma":
+    elif kernel in ("mfma", "mfma128"):
         ops.attention_prefill_mfma(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
-                                   bt.to(dev), i32(work_seq), i32(work_qoff), scale, window)
+                                   bt.to(dev), i32(work_seq), i32(work_qoff), scale, window, rows)
     else:
         assert all(ql == 1 for ql in q_lens)
         ops.attention_decode(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
@@ -275,16 +275,24 @@ def test_attention_decode_window(ops, dtype):
     dict(seq_lens=[129, 300], q_lens=[129, 65], Hq=4, Hkv=2, D=96, P=16),
     dict(seq_lens=[1, 2, 64, 65], q_lens=[1, 2, 64, 65], Hq=2, Hkv=2, D=64, P=4),
 ])
-def test_attention_prefill_mfma(ops, case):
-    _attention_case(ops, torch.bfloat16, kernel="mfma", **case)
+@pytest.mark.parametrize("kernel", ["mfma", "mfma128"])
+def test_attention_prefill_mfma(ops, case, kernel):
+    _attention_case(ops, torch.bfloat16, kernel=kernel, **case)
 
 
-def test_attention_prefill_mfma_window(ops):
+@pytest.mark.parametrize("kernel", ["mfma", "mfma128"])
+def test_attention_prefill_mfma_window(ops, kernel):
     _attention_case(ops, torch.bfloat16, seq_lens=[300, 90], q_lens=[150, 25], Hq=4, Hkv=2, D=64,
-                    P=8, window=70, kernel="mfma")
+                    P=8, window=70, kernel=kernel)
 
 
-@pytest.mark.parametrize("kernel", ["decode", "decode_mfma", "mfma"])
+def test_attention_prefill_mfma_long(ops):
+    """Many key tiles, a prefix in the cache, rows that end inside a block."""
+    _attention_case(ops, torch.bfloat16, seq_lens=[1100, 700], q_lens=[777, 300], Hq=4, Hkv=1, D=64,
+                    P=16, kernel="mfma128")
+
+
+@pytest.mark.parametrize("kernel", ["decode", "decode_mfma", "mfma", "mfma128"])
 def test_attention_far_key_stands_out_fast_kernels(ops, kernel):
     def boost(q, dk, kc, bt):
         direction = torch.ones(64) * 2.0
@@ -292,7 +300,7 @@ def test_attention_far_key_stands_out_fast_kernels(ops, kernel):
         page = int(bt[0, 0])
         kc[page, :, 3] = direction.to(kc.dtype)
         dk[0][3] = direction
-    ql = 2 if kernel == "mfma" else 1
+    ql = 2 if kernel.startswith("mfma") else 1
     _attention_case(ops, torch.bfloat16, seq_lens=[700], q_lens=[ql], Hq=2, Hkv=1, D=64, P=16,
                     boost=boost, kernel=kernel, splits=4)
 
