@@ -36,6 +36,20 @@ LLAMA_1B = {
 }
 
 
+SHAPES = {
+    "1b": {},
+    # Llama-3.2-3B shape
+    "3b": {"num_hidden_layers": 28, "hidden_size": 3072, "num_attention_heads": 24,
+           "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 8192},
+    # Llama-3.1-8B shape
+    "8b": {"num_hidden_layers": 32, "hidden_size": 4096, "num_attention_heads": 32,
+           "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 14336,
+           "tie_word_embeddings": False,
+           "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                            "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}},
+}
+
+
 def log(msg):
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
@@ -54,6 +68,49 @@ def model_numbers(cfg, dtype_bytes):
     }
 
 
+def mixed_workload(args, cfg, short):
+    """The secondary workload: a continuous batch of N requests with prompts of
+    128..4096 tokens, computed in 512-token portions beside the decodes of the
+    others, 256 greedy tokens each. Reports generated tokens per second of the
+    whole run and the prompt tokens per second that went in beside them."""
+    import torch
+    from pytriton_llama_amd.config import EngineConfig
+    from pytriton_llama_amd.engine import Engine, SamplingParams
+    N, new = args.mixed, 256
+    g = torch.Generator().manual_seed(99)
+    lens = torch.randint(128, 4097, (N,), generator=g).tolist()
+    page = 16
+    pages = sum(-(-(n + new + 8) // page) for n in lens) + 8
+    ec = EngineConfig(dtype=args.dtype, page_size=page, num_pages=pages, max_num_seqs=N,
+                      max_num_batched_tokens=512 + N, prefill_chunk=512, max_model_len=4096 + new + 8, seed=0)
+    t0 = time.time()
+    log(f"building the {cfg['num_hidden_layers']}-layer {args.shape} model with random weights ({args.dtype})")
+    engine = Engine(cfg, ec, random_seed=0)
+    log(f"model ready in {time.time() - t0:.1f}s")
+    sp = SamplingParams(temperature=0.0, max_new_tokens=new, ignore_eos=True)
+    warm = engine.generate([torch.randint(0, cfg["vocab_size"], (600,), generator=g).tolist()],
+                           SamplingParams(temperature=0.0, max_new_tokens=8, ignore_eos=True))
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lens]
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    steps = 0
+    for p in prompts:
+        engine.add_request(p, sp)
+    while engine.has_work:
+        engine.step()
+        steps += 1
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t
+    out = {"metric": f"mixed continuous batch, Llama {args.shape.upper()} shape: {N} requests, prompts 128..4096, "
+                     f"512-token portions beside decodes, {new} new tokens each",
+           "value": round(N * new / dt, 1), "unit": "generated tokens/s", "seconds": round(dt, 3),
+           "engine_steps": steps, "prompt_tokens": sum(lens),
+           "prompt_tokens_per_s": round(sum(lens) / dt, 1), "preemptions": engine.scheduler.num_preemptions,
+           "dtype": short, "data": "synthetic", "n_gpus": 1}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -66,6 +123,11 @@ def main():
     ap.add_argument("--points", default="1,64", help="other batch sizes to report, '' for none")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--prefill-only", action="store_true", help="measure the prefill and stop (for profiles)")
+    ap.add_argument("--shape", default="1b", choices=sorted(SHAPES),
+                    help="layer sizes: the default 1b is the benchmark; 3b and 8b are the secondary shapes")
+    ap.add_argument("--mixed", type=int, default=0, metavar="N",
+                    help="instead of the decode measurement: N requests with prompts of 128..4096 tokens "
+                         "through the scheduler in 512-token portions beside decodes, 256 new tokens each")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
@@ -76,6 +138,7 @@ def main():
     from pytriton_llama_amd.engine import Engine, SamplingParams
 
     cfg = dict(LLAMA_1B)
+    cfg.update(SHAPES[args.shape])
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -89,6 +152,8 @@ def main():
     # requests whose prompt is in first go on decoding while the others' prompts are computed
     slack = max_batch * -(-S // max(S, 2048)) + 8
     per_req_pages = -(-(S + W + K + slack) // page)
+    if args.mixed:
+        return mixed_workload(args, cfg, short)
     ec = EngineConfig(dtype=args.dtype, page_size=page, num_pages=per_req_pages * max_batch + 8,
                       max_num_seqs=max_batch, max_num_batched_tokens=max(S, 2048),
                       max_model_len=S + W + K + slack, seed=0)
@@ -162,16 +227,17 @@ def main():
         log(f"decode batch {b}: {r:.0f} tok/s, {st * 1e3:.3f} ms/step")
 
     out = {
-        "metric": f"decode tokens/s, Llama-3.2-1B shape, batch {args.batch}, {S}-token prompts",
+        "metric": f"decode tokens/s, Llama {args.shape.upper()} shape, batch {args.batch}, {S}-token prompts",
         "value": round(rate, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": short, "data": "synthetic",
         "config": {
-            "model": "Llama-3.2-1B shape, random weights N(0,0.02)", "layers": cfg["num_hidden_layers"],
+            "model": f"Llama {args.shape.upper()} shape, random weights N(0,0.02)", "layers": cfg["num_hidden_layers"],
             "layers_of_full_model": full_layers, "hidden_size": cfg["hidden_size"],
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate_size": cfg["intermediate_size"],
-            "vocab_size": cfg["vocab_size"], "tied_embeddings": True, "rope": "llama3 factor 32",
+            "vocab_size": cfg["vocab_size"], "tied_embeddings": cfg["tie_word_embeddings"],
+            "rope": f"llama3 factor {cfg['rope_scaling']['factor']:g}",
             "global_batch": args.batch, "seq_len": S, "context_at_timing": round(mean_ctx),
             "page_size": page, "kv_dtype": short, "sampling": "greedy", "parallelism": "single GPU",
         },

@@ -795,6 +795,11 @@ extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void
 // in ptl_attention_decode. Needs D % 32 == 0, D <= 128, Hq/Hkv <= 16.
 // ===========================================================================
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
+// 16-key tiles a wave has in flight per turn; measured on MI355X: 2 beats 4 (more
+// workgroups fit a CU) and 1 (more turns) from head size 64 to 128
+#ifndef DEC_UNR
+#define DEC_UNR(NDT) 2
+#endif
 
 template <int NDT>
 __global__ void __launch_bounds__(256)
@@ -815,7 +820,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
   const int ctx = ctx_len[seq];
   const int k_lo = window > 0 ? max(0, ctx - window) : 0;
   const int span = ctx - k_lo;
-  constexpr int UNR = NDT <= 2 ? 4 : 2;   // 16-key tiles a wave loads ahead
+  constexpr int UNR = DEC_UNR(NDT);       // 16-key tiles a wave loads ahead
   constexpr int TILE = 64 * UNR;          // keys per turn of the workgroup
   const int per_split = ((span + num_splits - 1) / num_splits + TILE - 1) / TILE * TILE;
   const int k_begin = k_lo + split * per_split;
@@ -978,7 +983,7 @@ static int launch_decode_mfma(void* out, long out_stride, const void* q, long q_
                               int page_size, int window, float scale, int num_splits,
                               hipStream_t stream) {
   constexpr int D = 32 * NDT;
-  constexpr int UNR = NDT <= 2 ? 4 : 2;
+  constexpr int UNR = DEC_UNR(NDT);
   dim3 grid(n_seq, Hkv, num_splits);
   const size_t lds_merge = (size_t)(4 * 16 * D + 4 * 16 * 2) * sizeof(float);
   const size_t lds_values = (size_t)4 * UNR * 16 * (D + 4) * sizeof(bf16_t);

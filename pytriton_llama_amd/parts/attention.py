@@ -96,7 +96,7 @@ class PagedAttention(Part):
         D = self.head_dim
         G = self.num_heads // self.num_kv_heads
         if matrix_cores:
-            turn = 256 if D <= 64 else 128          # keys a workgroup takes per turn
+            turn = 128                              # keys a workgroup takes per turn
             groups = self.num_kv_heads
         else:
             lpk = 1
@@ -107,7 +107,7 @@ class PagedAttention(Part):
         span = max(ctx.ctx_lens[:n_dec])
         if self.window:
             span = min(span, self.window)
-        want = -(-768 // max(1, n_dec * groups))
+        want = -(-1024 // max(1, n_dec * groups))       # about a thousand workgroups (measured)
         return max(1, min(want, -(-span // turn), 64))
 
     def attend(self, out, q, cache, ctx, group) -> None:
