@@ -77,4 +77,5 @@ def first_mismatch(got, want, tol):
     return None
 
 
-TOL = {torch.float32: 2e-4, torch.bfloat16: 4e-2}
+# measured on MI355X: float32 stays below 3e-6, bfloat16 below 3e-2 (tests/ tiny and wide models)
+TOL = {torch.float32: 2e-5, torch.bfloat16: 4e-2}
