@@ -20,14 +20,20 @@ class Architecture:
 
 
 MODEL_REGISTRY: Dict[str, Architecture] = {}
+# config.json files without an "architectures" entry are recognised by their model_type
+MODEL_TYPE_ALIASES: Dict[str, str] = {}
 
 
-def register_model(name: str, config_class, build) -> None:
+def register_model(name: str, config_class, build, model_type: str = None) -> None:
     MODEL_REGISTRY[name] = Architecture(name, config_class, build)
+    if model_type:
+        MODEL_TYPE_ALIASES[model_type] = name
 
 
 def architecture_of(config_dict: Dict[str, Any]) -> Architecture:
     archs = config_dict.get("architectures")
+    if not archs and config_dict.get("model_type") in MODEL_TYPE_ALIASES:
+        archs = [MODEL_TYPE_ALIASES[config_dict["model_type"]]]
     if not archs:
         raise ConfigError("config.json has no 'architectures' entry; "
                           f"supported: {sorted(MODEL_REGISTRY)}")

@@ -82,4 +82,4 @@ def build_llama(cfg: LlamaConfig) -> CausalLM:
                     ignorable)
 
 
-register_model("LlamaForCausalLM", LlamaConfig, build_llama)
+register_model("LlamaForCausalLM", LlamaConfig, build_llama, model_type="llama")

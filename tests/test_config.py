@@ -47,12 +47,21 @@ def test_kv_heads_default_to_heads():
     ({"vocab_size": None}, "vocab_size"),
     ({"hidden_size": 60, "num_attention_heads": 7}, "head_dim"),
     ({"architectures": ["GPT2LMHeadModel"]}, "not supported"),
-    ({"architectures": []}, "architectures"),
+    ({"architectures": [], "model_type": "other"}, "architectures"),
 ])
 def test_rejects_what_it_cannot_run(change, word):
     d = copy.deepcopy(TINY_A)
     d.update(change)
     with pytest.raises(ConfigError, match=word):
+        config_from_dict(d)
+
+
+def test_model_type_stands_in_for_a_missing_architectures_entry():
+    d = copy.deepcopy(TINY_A)
+    del d["architectures"]
+    assert isinstance(config_from_dict(d), LlamaConfig)
+    d["model_type"] = "gpt2"
+    with pytest.raises(ConfigError, match="architectures"):
         config_from_dict(d)
 
 
