@@ -209,3 +209,166 @@ extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int M
   if (M <= 32) return launch_skinny<2, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
   return launch_skinny<4, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
 }
+
+// ===========================================================================
+// Decode-step products with their follow-up fused in, for at most 16 rows of x:
+//
+// ptl_gate_up_silu_bf16:  out[m, c] = silu(x . Wg[c]) * (x . Wu[c])   (W = [Wg; Wu], [2I, K])
+// ptl_qkv_rope_store_bf16: q, k, v = x . Wqkv^T; q and k rotated by the angles
+//     positions[m] * inv_freq[j] on the pairs (j, j + D/2); q written out, the
+//     rotated k and v written into the cache pages at slots[m].
+//
+// Both are the skinny kernel above with two 16-row weight tiles per workgroup,
+// chosen so that the two values an output needs meet in one lane of the result
+// tile: gate row c with up row I + c; column j of a head with column j + D/2.
+// They replace a product, an element-wise kernel and the trip through memory
+// between them (lite_llama/models/llama.py:75-90 runs q_proj, kv_proj, the rotary
+// kernel and the cache copy one after the other; :120 gate, up, SwiGLU, down).
+// The projections are rounded to bfloat16 before the follow-up, as the unfused path
+// stores them, so both paths agree to the order of the sums.
+// ===========================================================================
+#define PAIR_SILU 0
+#define PAIR_ROPE 1
+
+struct RopeStoreArgs {
+  const int32_t* positions;   // [M]
+  const float* inv_freq;      // [D/2] or null: no rotation
+  const int32_t* slots;       // [M] or null: no store
+  bf16_t* k_cache;            // [pages, Hkv, page_size, D]
+  bf16_t* v_cache;
+  int Hq, Hkv, D, page_size;
+};
+
+template <int MODE, int U>
+__global__ void __launch_bounds__(1024)
+gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                 int M, int N_out, int K, long ldx, long ldy, int k_per_wave, int pair_offset,
+                 int tiles_per_group, int group_rows, RopeStoreArgs rs) {
+  extern __shared__ float red[];                 // [waves][2][64][4]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, lg = lane >> 4;
+  const int nwaves = blockDim.x >> 6;
+  // workgroup b takes tile (b % tiles_per_group) of group (b / tiles_per_group): rows
+  // r1 .. r1+15 and r1 + pair_offset .. of W. SiLU: one group, tiles over I. Rope: a
+  // group is a head (group_rows = D), its tiles cover the first half of the head.
+  const int group = blockIdx.x / tiles_per_group;
+  const int tile = blockIdx.x - group * tiles_per_group;
+  const int r1 = group * group_rows + 16 * tile;
+  const int r2 = r1 + pair_offset;
+  const bf16_t* wp1 = w + (size_t)(r1 + ln) * K + 8 * lg;
+  const bf16_t* wp2 = w + (size_t)(r2 + ln) * K + 8 * lg;
+  const bf16_t* xp = x + (size_t)min(ln, M - 1) * ldx + 8 * lg;
+  gs_f32x4_t acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+
+  const int kb = wave * k_per_wave;
+  const int ke = min(K, kb + k_per_wave);
+  for (int k = kb; k < ke; k += 32 * U) {
+    GsFrag w1[U], w2[U], xf[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = k + 32 * u;
+      const bool ok = kk + 8 * lg < ke;
+      w1[u].u = ok ? *reinterpret_cast<const uint4*>(wp1 + kk) : make_uint4(0, 0, 0, 0);
+      w2[u].u = ok ? *reinterpret_cast<const uint4*>(wp2 + kk) : make_uint4(0, 0, 0, 0);
+      xf[u].u = (ok && ln < M) ? *reinterpret_cast<const uint4*>(xp + kk) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, xf[u].v, acc1, 0, 0, 0);
+      acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2[u].v, xf[u].v, acc2, 0, 0, 0);
+    }
+  }
+  if (nwaves > 1) {
+    *reinterpret_cast<gs_f32x4_t*>(red + (((size_t)wave * 2 + 0) * 64 + lane) * 4) = acc1;
+    *reinterpret_cast<gs_f32x4_t*>(red + (((size_t)wave * 2 + 1) * 64 + lane) * 4) = acc2;
+    __syncthreads();
+    if (wave != 0) return;
+    for (int wv = 1; wv < nwaves; ++wv) {
+      acc1 += *reinterpret_cast<const gs_f32x4_t*>(red + (((size_t)wv * 2 + 0) * 64 + lane) * 4);
+      acc2 += *reinterpret_cast<const gs_f32x4_t*>(red + (((size_t)wv * 2 + 1) * 64 + lane) * 4);
+    }
+  }
+  const int m = ln;                 // the result tiles hold rows 4*lg+i of W, column m of x^T
+  if (m >= M) return;
+  if (MODE == PAIR_SILU) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = r1 + 4 * lg + i;
+      // the gate and up products are rounded to bfloat16 as the unfused path stores them
+      const float g = round_to<bf16_t>(acc1[i]), u = round_to<bf16_t>(acc2[i]);
+      if (c < N_out) y[(size_t)m * ldy + c] = float_to_bf16(g / (1.0f + expf(-g)) * u);
+    }
+  } else {
+    const int D = rs.D, half = D >> 1;
+    const int head = group;                      // 0..Hq-1: q; then Hkv k heads; then Hkv v heads
+    const bool is_q = head < rs.Hq, is_k = !is_q && head < rs.Hq + rs.Hkv;
+    const float pos = (float)rs.positions[m];
+    const int slot = rs.slots ? rs.slots[m] : -1;
+    bf16_t* dst = nullptr;
+    if (is_q) {
+      dst = y + (size_t)m * ldy + (size_t)head * D;
+    } else if (slot >= 0) {
+      const int kvh = is_k ? head - rs.Hq : head - rs.Hq - rs.Hkv;
+      const int page = slot / rs.page_size, off = slot - page * rs.page_size;
+      dst = (is_k ? rs.k_cache : rs.v_cache) + (((size_t)page * rs.Hkv + kvh) * rs.page_size + off) * D;
+    }
+    if (dst == nullptr) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = 16 * tile + 4 * lg + i;      // column in the first half of the head
+      // as in the unfused path, the projection is rounded to bfloat16 before the rotation
+      float x1 = round_to<bf16_t>(acc1[i]), x2 = round_to<bf16_t>(acc2[i]);
+      if ((is_q || is_k) && rs.inv_freq) {
+        float sn, cs;
+        sincosf(pos * rs.inv_freq[j], &sn, &cs);
+        const float o1 = x1 * cs - x2 * sn, o2 = x2 * cs + x1 * sn;
+        x1 = o1; x2 = o2;
+      }
+      dst[j] = float_to_bf16(x1);
+      dst[j + half] = float_to_bf16(x2);
+    }
+  }
+}
+
+static int pair_waves(int blocks, int K) {
+  int waves = 1;
+  while (waves < 16 && (long)blocks * waves < 4096 && K / (waves * 2) >= 256) waves <<= 1;
+  if (waves < 4 && K >= 1024) waves = 4;
+  return waves;
+}
+
+// out [M, I] = silu(x Wg^T) * (x Wu^T) for W = [Wg; Wu] of shape [2I, K]; M <= 16, I % 16 == 0
+extern "C" int ptl_gate_up_silu_bf16(void* out, const void* x, const void* w, int M, int I, int K,
+                                     long ldx, hipStream_t stream) {
+  if (M <= 0 || I <= 0) return PTL_OK;
+  if (M > 16 || I % 16 || K <= 0 || K % 8 || ldx % 8 || ldx < K) return PTL_ERR_ARG;
+  const int blocks = I / 16;
+  const int waves = pair_waves(blocks, K);
+  const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
+  const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
+  RopeStoreArgs none = {};
+  gemm_pair_kernel<PAIR_SILU, 8><<<blocks, waves * 64, lds, stream>>>(
+      (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, I, K, ldx, I, k_per_wave, I, blocks, 0, none);
+  return ptl_launch_status();
+}
+
+// q_out [M, Hq, D] (row stride ldq); w [(Hq + 2 Hkv) D, K] rows q | k | v; M <= 16, D % 32 == 0
+extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, const void* w, int M,
+                                       int K, long ldx, const int32_t* positions,
+                                       const float* inv_freq, const int32_t* slots, void* k_cache,
+                                       void* v_cache, int Hq, int Hkv, int D, int page_size,
+                                       hipStream_t stream) {
+  if (M <= 0) return PTL_OK;
+  if (M > 16 || Hq <= 0 || Hkv <= 0 || D <= 0 || D % 32 || K <= 0 || K % 8 || ldx % 8 || ldx < K ||
+      ldq < (long)Hq * D || page_size <= 0 || !positions || (slots && (!k_cache || !v_cache)))
+    return PTL_ERR_ARG;
+  const int tiles = D / 32;                       // 16-wide tiles in half a head
+  const int blocks = (Hq + 2 * Hkv) * tiles;
+  const int waves = pair_waves(blocks, K);
+  const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
+  const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
+  RopeStoreArgs rs = {positions, inv_freq, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, Hq, Hkv, D, page_size};
+  gemm_pair_kernel<PAIR_ROPE, 8><<<blocks, waves * 64, lds, stream>>>(
+      (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,
+      tiles, D, rs);
+  return ptl_launch_status();
+}

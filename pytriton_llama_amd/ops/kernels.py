@@ -210,6 +210,80 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     return y
 
 
+FUSED_MAX_ROWS = 16
+
+
+def _fused_x_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
+            and 0 < x.shape[0] <= FUSED_MAX_ROWS and x.shape[1] % 8 == 0 and x.stride(1) == 1
+            and (x.shape[0] == 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0
+            and w.is_contiguous() and w.data_ptr() % 16 == 0 and w.shape[1] == x.shape[1])
+
+
+def gate_up_silu_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return _fused_x_ok(x, w) and w.shape[0] % 32 == 0
+
+
+def gate_up_silu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """silu(x Wg^T) * (x Wu^T) for w = [Wg; Wu] ([2I, K]) and at most 16 rows of
+    bfloat16 x, in one kernel (see csrc/gemm.hip)."""
+    if not gate_up_silu_fits(x, w):
+        raise KernelError("gate_up_silu: needs bfloat16, at most 16 rows, K a multiple of 8, "
+                          "I a multiple of 16, aligned rows")
+    M, K = x.shape
+    I = w.shape[0] // 2
+    out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+    lib = library.load("gemm")
+    _check(lib.ptl_gate_up_silu_bf16(_ptr(out), _ptr(x), _ptr(w), M, I, K,
+                                     ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)), _stream()),
+           "gate_up_silu")
+    return out
+
+
+def qkv_rope_store_fits(x: torch.Tensor, w: torch.Tensor, head_dim: int) -> bool:
+    return _fused_x_ok(x, w) and head_dim % 32 == 0
+
+
+def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
+                   inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                   num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
+    """q, k, v = x @ w.T (rows of w: q | k | v), q and k rotated, k and v written
+    into the cache pages at ``slots``; returns the rotated q [M, Hq, D]. At most 16
+    rows of bfloat16 x, head sizes in steps of 32 (see csrc/gemm.hip)."""
+    if not qkv_rope_store_fits(x, w, head_dim):
+        raise KernelError("qkv_rope_store: needs bfloat16, at most 16 rows, K a multiple of 8, "
+                          "a head size in steps of 32, aligned rows")
+    M, K = x.shape
+    Hq, Hkv, D = num_heads, num_kv_heads, head_dim
+    if w.shape[0] != (Hq + 2 * Hkv) * D:
+        raise KernelError(f"qkv_rope_store: weight has {w.shape[0]} rows, "
+                          f"({Hq} + 2*{Hkv}) * {D} expected")
+    _need_gpu(positions, inv_freq, slots, k_cache, v_cache)
+    _i32(positions, "positions")
+    if positions.numel() != M:
+        raise KernelError("qkv_rope_store: one position per row of x")
+    if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != D // 2
+                                 or not inv_freq.is_contiguous()):
+        raise KernelError(f"qkv_rope_store: inv_freq must be float32 [{D // 2}]")
+    if slots is not None:
+        if slots.dtype != torch.int32 or slots.numel() != M or not slots.is_contiguous():
+            raise KernelError("qkv_rope_store: slots must be contiguous int32 [M]")
+        for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+            if c is None or c.dim() != 4 or c.shape[1:] != (Hkv, page_size, D) \
+                    or c.dtype != torch.bfloat16 or not c.is_contiguous():
+                raise KernelError(f"qkv_rope_store: {name} must be contiguous bfloat16 "
+                                  f"[pages, {Hkv}, {page_size}, {D}]")
+    q = torch.empty((M, Hq, D), dtype=torch.bfloat16, device=x.device)
+    lib = library.load("gemm")
+    _check(lib.ptl_qkv_rope_store_bf16(
+        _ptr(q), ctypes.c_long(Hq * D), _ptr(x), _ptr(w), M, K,
+        ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)), _ptr(positions), _ptr(inv_freq),
+        _ptr(slots), _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D, int(page_size), _stream()),
+        "qkv_rope_store")
+    return q
+
+
 def attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                       block_table: torch.Tensor, work_seq: torch.Tensor, work_qoff: torch.Tensor,

@@ -70,6 +70,16 @@ class PagedAttention(Part):
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         T = x.shape[0]
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
+        group = ctx.groups[cache.group]
+        rotary = self.position.rotary_inv_freq() if self.position is not None else None
+        if (self.position is None or rotary is not None) and ops.qkv_rope_store_fits(x, self.qkv, D):
+            # the few rows of a decode step: projection, rotation and cache write in one kernel
+            q = ops.qkv_rope_store(x, self.qkv, ctx.positions, rotary,
+                                   group.slots if cache.writable else None, cache.k, cache.v,
+                                   Hq, Hkv, D, cache.page_size)
+            out = torch.empty((T, Hq, D), dtype=x.dtype, device=x.device)
+            self.attend(out, q, cache, ctx, group)
+            return linear(out.view(T, Hq * D), self.o)
         qkv = linear(x, self.qkv)
         q = qkv[:, :self.q_size].view(T, Hq, D)
         k = qkv[:, self.q_size:self.q_size + self.kv_size].view(T, Hkv, D)
@@ -79,7 +89,6 @@ class PagedAttention(Part):
             inv_freq = self.position.rotary_inv_freq()
             if inv_freq is None:
                 self.position.apply(q, k, ctx.positions)
-        group = ctx.groups[cache.group]
         ops.rope_store(q, k, v, ctx.positions, inv_freq,
                        group.slots if cache.writable else None, cache.k, cache.v,
                        cache.page_size)

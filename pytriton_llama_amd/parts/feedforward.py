@@ -38,4 +38,7 @@ class SwiGLU(Part):
         self.down = place(tensors[d], "matrix", dtype, device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if ops.gate_up_silu_fits(x, self.gate_up):
+            # the few rows of a decode step: product and SiLU-multiply in one kernel
+            return linear(ops.gate_up_silu(x, self.gate_up), self.down)
         return linear(ops.silu_mul(linear(x, self.gate_up)), self.down)

@@ -105,6 +105,58 @@ def test_gemm_skinny(ops, out_dtype, mnk):
         ops.gemm_skinny(x[:, :K - 4], w[:, :K - 4].contiguous())
 
 
+@pytest.mark.parametrize("mik", [(1, 176, 64), (8, 8192, 2048), (16, 320, 136), (5, 48, 2056)])
+def test_gate_up_silu(ops, mik):
+    M, I, K = mik
+    torch.manual_seed(8)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(2 * I, K, device="cuda") / math.sqrt(K) * 2).to(torch.bfloat16)
+    got = ops.gate_up_silu(x, w)
+    want = ops.silu_mul(ops.gemm_nt(x, w))              # the unfused kernels
+    torch.testing.assert_close(got.float(), want.float(), atol=2e-2, rtol=2e-2)
+    gu = (x.double() @ w.double().T).float()
+    plain = plain_llama.silu(gu[:, :I]) * gu[:, I:]
+    torch.testing.assert_close(got.float(), plain, atol=3e-2, rtol=3e-2)
+    with pytest.raises(ops.KernelError):
+        ops.gate_up_silu(torch.zeros(17, K, device="cuda", dtype=torch.bfloat16), w)
+
+
+@pytest.mark.parametrize("dims", [(4, 2, 64, 16, 72), (3, 1, 32, 4, 128), (8, 8, 128, 16, 2048), (6, 3, 96, 5, 200)])
+def test_qkv_rope_store(ops, dims):
+    Hq, Hkv, D, P, K = dims
+    M = 7
+    torch.manual_seed(9)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn((Hq + 2 * Hkv) * D, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    positions = torch.tensor([0, 1, 5, 77, 1000, 4095, 100000], dtype=torch.int32, device="cuda")
+    inv_freq = plain_llama.rope_inv_freq_default(500000.0, D).cuda()
+    pages = 5
+    slots = torch.randperm(pages * P)[:M].to(torch.int32).cuda()
+    slots[3] = -1                                           # this row's keys are not stored
+    kc = torch.zeros(pages, Hkv, P, D, device="cuda", dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    q = ops.qkv_rope_store(x, w, positions, inv_freq, slots, kc, vc, Hq, Hkv, D, P)
+    # the unfused kernels on the same inputs
+    qkv = ops.gemm_nt(x, w)
+    q2 = qkv[:, :Hq * D].view(M, Hq, D)
+    k2 = qkv[:, Hq * D:(Hq + Hkv) * D].view(M, Hkv, D)
+    v2 = qkv[:, (Hq + Hkv) * D:].view(M, Hkv, D)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ops.rope_store(q2, k2, v2, positions, inv_freq, slots, kc2, vc2, P)
+    torch.testing.assert_close(q.float(), q2.float(), atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(kc.float(), kc2.float(), atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(vc.float(), vc2.float(), atol=2e-2, rtol=2e-2)
+    assert torch.all(kc.view(pages, Hkv, P, D)[:, :, :, :].sum() != 0)
+    # and the plain formulas
+    full = (x.double() @ w.double().T).float().cpu()
+    cos, sin = plain_llama.rope_cos_sin(inv_freq.cpu(), positions.cpu())
+    want_q = plain_llama.apply_rope(full[:, :Hq * D].view(M, Hq, D), cos, sin)
+    torch.testing.assert_close(q.float().cpu(), want_q, atol=3e-2, rtol=3e-2)
+    # without rotation and without a store
+    q3 = ops.qkv_rope_store(x, w, positions, None, None, None, None, Hq, Hkv, D, P)
+    torch.testing.assert_close(q3.float().cpu(), full[:, :Hq * D].view(M, Hq, D), atol=3e-2, rtol=3e-2)
+
+
 def _rope_reference(x, positions, inv_freq):
     cos, sin = plain_llama.rope_cos_sin(inv_freq, positions)
     return plain_llama.apply_rope(x, cos, sin)
