@@ -449,9 +449,9 @@ def sample_top_p(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.T
         if t.dtype != torch.float32 or t.numel() != R or not t.is_contiguous():
             raise KernelError(f"sample_top_p: {name} must be float32 [{R}]")
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-    probs = torch.empty((R, V), dtype=torch.float32, device=logits.device) if return_probs else None
+    probs = torch.empty((R, V), dtype=torch.float32, device=logits.device)   # scratch, then result
     lib = library.load("sampling")
-    _check(lib.ptl_sample_top_p(_ptr(out), _ptr(probs), _ptr(logits), R, V,
+    _check(lib.ptl_sample_top_p(_ptr(out), _ptr(probs), int(return_probs), _ptr(logits), R, V,
                                 ctypes.c_long(logits.stride(0)), _ptr(temperature), _ptr(top_p),
                                 _ptr(uniform), _stream()), "sample_top_p")
     return (out, probs) if return_probs else out

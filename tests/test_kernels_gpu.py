@@ -449,3 +449,34 @@ def test_kernels_refuse_cpu_tensors(ops):
         ops.silu_mul(torch.zeros(2, 4))
     with pytest.raises(ops.KernelError):
         ops.add_rmsnorm(torch.zeros(2, 20000, device="cuda"), None, torch.ones(20000, device="cuda"), 1e-5)
+
+
+def test_sample_top_p_large_vocabulary_and_ties(ops):
+    """At vocabulary size, with a peaked and a flat row, and a row of many equal
+    logits (more tokens in one histogram bin than the kernel gathers)."""
+    torch.manual_seed(11)
+    V = 128256
+    logits = torch.randn(4, V)
+    logits[0] *= 4.0                                   # peaked
+    logits[1] *= 0.05                                  # nearly flat
+    logits[2] = 0.0                                    # all equal but a few
+    logits[2, [5, 77, 99999]] = torch.tensor([3.0, 2.0, 1.0])
+    logits[3, 1234] = 40.0                             # one token holds all the mass
+    t = torch.tensor([0.8, 1.0, 1.0, 0.6])
+    p = torch.tensor([0.9, 0.5, 0.5, 0.9])
+    u = torch.tensor([0.3, 0.9, 0.999999, 0.5])
+    tok, probs = ops.sample_top_p(logits.cuda(), t.cuda(), p.cuda(), u.cuda(), return_probs=True)
+    for r in (0, 1, 3):
+        want = plain_llama.top_p_probs(logits[r], float(t[r]), float(p[r]))
+        got = probs[r].cpu().double()
+        # the nucleus may differ by a token or two at its edge where the float32 running
+        # mass meets top_p; the mass that changes hands is tiny
+        assert float((got - want).abs().sum()) < 1e-3
+        assert want[int(tok[r])] > 0
+    assert int(tok[3]) == 1234
+    # equal logits are kept or dropped together: the three larger ones first, then all or none
+    got2 = probs[2].cpu()
+    assert got2[5] > got2[77] > got2[99999] > 0
+    rest = got2[torch.arange(V)[(torch.arange(V) != 5) & (torch.arange(V) != 77) & (torch.arange(V) != 99999)]]
+    assert float(rest.min()) == float(rest.max())
+    assert abs(float(got2.sum()) - 1) < 1e-4
