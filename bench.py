@@ -50,6 +50,9 @@ SHAPES = {
 }
 
 
+SHAPE_NAMES = {"1b": "Llama-3.2-1B", "3b": "Llama-3.2-3B", "8b": "Llama-3.1-8B"}
+
+
 def log(msg):
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
@@ -101,7 +104,7 @@ def mixed_workload(args, cfg, short):
         steps += 1
     torch.cuda.synchronize()
     dt = time.perf_counter() - t
-    out = {"metric": f"mixed continuous batch, Llama {args.shape.upper()} shape: {N} requests, prompts 128..4096, "
+    out = {"metric": f"mixed continuous batch, {SHAPE_NAMES[args.shape]} shape: {N} requests, prompts 128..4096, "
                      f"512-token portions beside decodes, {new} new tokens each",
            "value": round(N * new / dt, 1), "unit": "generated tokens/s", "seconds": round(dt, 3),
            "engine_steps": steps, "prompt_tokens": sum(lens),
@@ -227,12 +230,12 @@ def main():
         log(f"decode batch {b}: {r:.0f} tok/s, {st * 1e3:.3f} ms/step")
 
     out = {
-        "metric": f"decode tokens/s, Llama {args.shape.upper()} shape, batch {args.batch}, {S}-token prompts",
+        "metric": f"decode tokens/s, {SHAPE_NAMES[args.shape]} shape, batch {args.batch}, {S}-token prompts",
         "value": round(rate, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": short, "data": "synthetic",
         "config": {
-            "model": f"Llama {args.shape.upper()} shape, random weights N(0,0.02)", "layers": cfg["num_hidden_layers"],
+            "model": f"{SHAPE_NAMES[args.shape]} shape, random weights N(0,0.02)", "layers": cfg["num_hidden_layers"],
             "layers_of_full_model": full_layers, "hidden_size": cfg["hidden_size"],
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate_size": cfg["intermediate_size"],
