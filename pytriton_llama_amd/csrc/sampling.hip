@@ -346,3 +346,31 @@ extern "C" int ptl_sample_top_p(int32_t* out, float* work, int want_probs, const
                                                      temperature, top_p, uniform);
   return ptl_launch_status();
 }
+
+// ptl_token_logprob: out[r] = log_softmax(logits[r])[tokens[r]], the log-probability the
+// reference reports for a generated token (F.log_softmax of the step's logits gathered at
+// the token, lite_llama/generete_with_probs.py:154-165). One workgroup a row.
+__global__ void __launch_bounds__(1024)
+token_logprob_kernel(float* __restrict__ out, const float* __restrict__ logits,
+                     const int32_t* __restrict__ tokens, int V, long stride) {
+  __shared__ float scratch[16];
+  const float* row = logits + (size_t)blockIdx.x * stride;
+  float mx = -INFINITY;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, row[i]);
+  mx = block_max(mx, scratch);
+  float z = 0.f;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) z += expf(row[i] - mx);
+  z = block_sum(z, scratch);
+  if (threadIdx.x == 0) {
+    const int t = tokens[blockIdx.x];
+    out[blockIdx.x] = (t >= 0 && t < V) ? row[t] - mx - logf(z) : -INFINITY;
+  }
+}
+
+extern "C" int ptl_token_logprob(float* out, const float* logits, const int32_t* tokens, int R, int V,
+                                 long stride, hipStream_t stream) {
+  if (R <= 0) return PTL_OK;
+  if (V <= 0 || stride < V) return PTL_ERR_ARG;
+  token_logprob_kernel<<<R, 1024, 0, stream>>>(out, logits, tokens, V, stride);
+  return ptl_launch_status();
+}

@@ -92,7 +92,13 @@ class Engine:
                 samplers.append(e.request)
         logits = self.runner.step(entries)
         tokens = self.sampler.sample(logits, samplers)
+        logprobs = self.sampler.logprobs(logits, samplers, tokens)
         outs = self.scheduler.update(plan, {r.id: t for r, t in zip(samplers, tokens)})
+        by_id = {r.id: lp for r, lp in zip(samplers, logprobs) if lp is not None}
+        for o in outs:
+            if o.request in by_id:
+                o.logprob = by_id[o.request]
+                self.requests[o.request].output_logprobs.append(o.logprob)
         return outs
 
     @property
@@ -103,10 +109,15 @@ class Engine:
     def generate(self, prompts: Sequence[Sequence[int]],
                  params: Union[SamplingParams, Sequence[SamplingParams], None] = None) -> List[List[int]]:
         """Generated token ids (without the prompt) for every prompt."""
+        return [r.output for r in self.generate_requests(prompts, params)]
+
+    def generate_requests(self, prompts, params=None) -> List[Request]:
+        """As ``generate``, returning the finished requests (tokens, log-probabilities,
+        finish reasons)."""
         ids = self._add_all(prompts, params)
         while self.has_work:
             self.step()
-        return [self.requests.pop(i).output for i in ids]
+        return [self.requests.pop(i) for i in ids]
 
     def generate_stream(self, prompts, params=None) -> Iterator[List[StepOutput]]:
         """Yields, step by step, the new token of every request that got one;
@@ -115,7 +126,7 @@ class Engine:
         index = {rid: i for i, rid in enumerate(ids)}
         while self.has_work:
             outs = self.step()
-            mine = [StepOutput(index[o.request], o.token, o.finished, o.finish_reason)
+            mine = [StepOutput(index[o.request], o.token, o.finished, o.finish_reason, o.logprob)
                     for o in outs if o.request in index]
             if mine:
                 yield mine

@@ -16,6 +16,7 @@ class SamplingParams:
     max_new_tokens: int = 128
     seed: Optional[int] = None        # None: derived from the engine seed and the request id
     ignore_eos: bool = False
+    logprobs: bool = False            # report log_softmax(logits)[token] of every generated token
 
     def __post_init__(self):
         if self.temperature < 0:
@@ -35,6 +36,7 @@ class Request:
     prompt: List[int]
     params: SamplingParams
     output: List[int] = field(default_factory=list)
+    output_logprobs: List[float] = field(default_factory=list)
     num_computed: int = 0             # tokens of prompt+output whose keys are in the cache
     status: str = WAITING
     finish_reason: Optional[str] = None
@@ -69,3 +71,4 @@ class StepOutput:
     token: int
     finished: bool
     finish_reason: Optional[str] = None
+    logprob: Optional[float] = None

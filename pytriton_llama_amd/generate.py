@@ -57,23 +57,28 @@ class GenerateText:
         self.model_config = self.engine.model.config
         self.tokenizer = load_tokenizer(tokenizer_path or checkpoints_dir)
 
-    def _params(self, max_gen_len, temperature, top_p, n_prompt):
+    def _params(self, max_gen_len, temperature, top_p, n_prompt, logprobs=False):
         room = self.engine_config.max_model_len - n_prompt
         if room < 1:
             raise ValueError(f"a prompt of {n_prompt} tokens leaves no room under max_seq_len "
                              f"{self.engine_config.max_model_len}")
         return SamplingParams(temperature=temperature, top_p=top_p,
-                              max_new_tokens=max(1, min(max_gen_len, room)))
+                              max_new_tokens=max(1, min(max_gen_len, room)), logprobs=logprobs)
 
     def generate(self, prompt_tokens: List[List[int]], max_gen_len: int, temperature: float = 0.6,
-                 top_p: float = 0.9, echo: bool = False) -> Tuple[List[List[int]], None]:
+                 top_p: float = 0.9, echo: bool = False, logprobs: bool = False
+                 ) -> Tuple[List[List[int]], Optional[List[List[float]]]]:
         """Token ids generated for every prompt (with the prompt in front when
-        ``echo``); generation of a request stops at its EOS token."""
-        params = [self._params(max_gen_len, temperature, top_p, len(p)) for p in prompt_tokens]
-        outs = self.engine.generate(prompt_tokens, params)
+        ``echo``); generation of a request stops at its EOS token. With ``logprobs``
+        the second result holds log_softmax(logits)[token] of every generated token
+        (the reference's generete_with_probs.py:89-97,154-165; prompt tokens under
+        ``echo`` have none and are not listed)."""
+        params = [self._params(max_gen_len, temperature, top_p, len(p), logprobs) for p in prompt_tokens]
+        reqs = self.engine.generate_requests(prompt_tokens, params)
+        outs = [r.output for r in reqs]
         if echo:
             outs = [list(p) + o for p, o in zip(prompt_tokens, outs)]
-        return outs, None
+        return outs, ([r.output_logprobs for r in reqs] if logprobs else None)
 
     def _need_tokenizer(self):
         if self.tokenizer is None:

@@ -455,3 +455,19 @@ def sample_top_p(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.T
                                 ctypes.c_long(logits.stride(0)), _ptr(temperature), _ptr(top_p),
                                 _ptr(uniform), _stream()), "sample_top_p")
     return (out, probs) if return_probs else out
+
+
+def token_logprob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+    """log_softmax(logits[r])[tokens[r]] for float32 logits [R, V] and int32 tokens [R]."""
+    _need_gpu(logits, tokens)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("token_logprob: logits must be float32 [R, V] with dense rows")
+    _i32(tokens, "tokens")
+    R, V = logits.shape
+    if tokens.numel() != R:
+        raise KernelError("token_logprob: one token per row")
+    out = torch.empty((R,), dtype=torch.float32, device=logits.device)
+    lib = library.load("sampling")
+    _check(lib.ptl_token_logprob(_ptr(out), _ptr(logits), _ptr(tokens), R, V,
+                                 ctypes.c_long(logits.stride(0)), _stream()), "token_logprob")
+    return out

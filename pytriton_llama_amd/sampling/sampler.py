@@ -28,6 +28,21 @@ class Sampler:
     def __init__(self, seed: int = 0):
         self.seed = int(seed)
 
+    def logprobs(self, logits: torch.Tensor, requests: Sequence[Request], tokens: Sequence[int]):
+        """log_softmax(logits)[token] for the requests that ask for it (None for the others),
+        from the unscaled logits as the reference does
+        (lite_llama/generete_with_probs.py:154-165)."""
+        want = [i for i, r in enumerate(requests) if r.params.logprobs]
+        out = [None] * len(requests)
+        if not want:
+            return out
+        rows = logits if len(want) == len(requests) else logits.index_select(
+            0, torch.tensor(want, dtype=torch.int32, device=logits.device))
+        toks = torch.tensor([tokens[i] for i in want], dtype=torch.int32, device=logits.device)
+        for i, lp in zip(want, ops.token_logprob(rows, toks).tolist()):
+            out[i] = lp
+        return out
+
     def sample(self, logits: torch.Tensor, requests: Sequence[Request]) -> List[int]:
         """logits float32 [R, V], row i for requests[i]; returns R token ids."""
         R = len(requests)

@@ -168,3 +168,21 @@ def test_decode_graphs_match_eager_steps(folder_b, dtype):
             both([("b", 9)])                              # a new request in the freed pages
     assert graphed.graphs.buckets[4].graph is not None and graphed.graphs.buckets[1].graph is not None
     assert replays == 40
+
+
+def test_logprobs_of_generated_tokens(folder_a):
+    """log_softmax of the plain logits at the tokens the engine chose."""
+    from pytriton_llama_amd.generate import GenerateText
+    folder, page = folder_a
+    cfg, w = plain_llama.read_model_folder(folder)
+    prompts = prompts_a()[:2]
+    gen = GenerateText(folder, max_seq_len=64, max_gpu_num_blocks=64, dtype="float32", page_size=page,
+                       max_batch_size=4)
+    toks, lps = gen.generate(prompts, max_gen_len=5, temperature=0.0, logprobs=True)
+    assert gen.generate(prompts, max_gen_len=5, temperature=0.0)[1] is None
+    for p, t, lp in zip(prompts, toks, lps):
+        assert len(lp) == len(t) == 5
+        for i in range(5):
+            logits = plain_llama.forward(cfg, w, list(p) + t[:i])[-1]
+            want = float(torch.log_softmax(logits.double(), -1)[t[i]])
+            assert abs(lp[i] - want) < 1e-4
