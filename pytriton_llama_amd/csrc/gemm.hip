@@ -7,6 +7,7 @@
 // matrix path of the true 32-bit mode (no reduced-precision matrix mode can
 // hide in it) and the fallback of the bfloat16 mode.
 #include "common.h"
+#include <stdlib.h>
 
 #define TM 64
 #define TN 64
@@ -115,15 +116,18 @@ union GsFrag {
   gs_bf16x8_t v;
 };
 
-template <int MT, int U, typename TY>
+// ROWS: weight rows a workgroup owns: 16 fill the MFMA tile; 8 (half the tile idle) give twice
+// the workgroups when N is so small that 16-row tiles would leave CUs without work.
+template <int MT, int U, int ROWS, typename TY>
 __global__ void __launch_bounds__(1024)
 gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                    int M, int N, int K, long ldx, long ldy, int k_per_wave) {
   extern __shared__ float red[];                 // [waves][MT][64][4]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, lg = lane >> 4;
   const int nwaves = blockDim.x >> 6;
-  const int n0 = blockIdx.x * 16;
-  const bf16_t* wp = w + (size_t)min(n0 + ln, N - 1) * K + 8 * lg;
+  const int n0 = blockIdx.x * ROWS;
+  const bool wrow = ln < ROWS;
+  const bf16_t* wp = w + (size_t)min(n0 + min(ln, ROWS - 1), N - 1) * K + 8 * lg;
   const bf16_t* xp[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) xp[t] = x + (size_t)min(16 * t + ln, M - 1) * ldx + 8 * lg;
@@ -139,7 +143,7 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
     for (int u = 0; u < U; ++u) {
       const int kk = k + 32 * u;
       const bool ok = kk + 8 * lg < ke;
-      wf[u].u = ok ? *reinterpret_cast<const uint4*>(wp + kk) : make_uint4(0, 0, 0, 0);
+      wf[u].u = (ok && wrow) ? *reinterpret_cast<const uint4*>(wp + kk) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < MT; ++t)   // columns past the last row of x are never stored: no load
         xf[t][u].u = (ok && 16 * t + ln < M) ? *reinterpret_cast<const uint4*>(xp[t] + kk)
@@ -172,15 +176,15 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int n = n0 + 4 * lg + i;
-      if (n < N) y[(size_t)m * ldy + n] = from_float<TY>(acc[t][i]);
+      if (4 * lg + i < ROWS && n < N) y[(size_t)m * ldy + n] = from_float<TY>(acc[t][i]);
     }
   }
 }
 
-template <int MT, int U>
-static int launch_skinny(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
-                         long ldy, int out_dtype, hipStream_t stream) {
-  const int blocks = (N + 15) / 16;
+template <int MT, int U, int ROWS>
+static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
+                              long ldy, int out_dtype, hipStream_t stream) {
+  const int blocks = (N + ROWS - 1) / ROWS;
   // enough waves to keep every SIMD of 256 CUs busy a few times over, each with
   // at least 256 elements of K to stream
   // (measured on MI355X: 4 waves a workgroup are best from N = 2048 to N = 128256 at
@@ -191,12 +195,22 @@ static int launch_skinny(void* y, const void* x, const void* w, int M, int N, in
   int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * MT * 64 * 4 * sizeof(float) : 0;
   if (out_dtype == PTL_DTYPE_F32)
-    gemm_skinny_kernel<MT, U, float><<<blocks, waves * 64, lds, stream>>>(
+    gemm_skinny_kernel<MT, U, ROWS, float><<<blocks, waves * 64, lds, stream>>>(
         (float*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave);
   else
-    gemm_skinny_kernel<MT, U, bf16_t><<<blocks, waves * 64, lds, stream>>>(
+    gemm_skinny_kernel<MT, U, ROWS, bf16_t><<<blocks, waves * 64, lds, stream>>>(
         (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave);
   return ptl_launch_status();
+}
+
+template <int MT, int U>
+static int launch_skinny(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
+                         long ldy, int out_dtype, hipStream_t stream) {
+  // measured on MI355X at K = 2048 and 8192: N = 2048 (128 tiles of 16 rows) gains 10 to 20 %
+  // from 8-row tiles, N = 3072 (192 tiles) loses
+  if ((N + 15) / 16 <= 160)
+    return launch_skinny_rows<MT, U, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
+  return launch_skinny_rows<MT, U, 16>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
 }
 
 extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int M, int N, int K,
