@@ -253,7 +253,7 @@ struct RopeStoreArgs {
   int Hq, Hkv, D, page_size;
 };
 
-template <int MODE, int U>
+template <int MODE, int U, int ROWS>
 __global__ void __launch_bounds__(1024)
 gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                  int M, int N_out, int K, long ldx, long ldy, int k_per_wave, int pair_offset,
@@ -266,10 +266,12 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   // group is a head (group_rows = D), its tiles cover the first half of the head.
   const int group = blockIdx.x / tiles_per_group;
   const int tile = blockIdx.x - group * tiles_per_group;
-  const int r1 = group * group_rows + 16 * tile;
+  // (ROWS = 8: half of the MFMA tile idle, twice the workgroups, for products with few rows)
+  const int r1 = group * group_rows + ROWS * tile;
   const int r2 = r1 + pair_offset;
-  const bf16_t* wp1 = w + (size_t)(r1 + ln) * K + 8 * lg;
-  const bf16_t* wp2 = w + (size_t)(r2 + ln) * K + 8 * lg;
+  const bool wrow = ln < ROWS;
+  const bf16_t* wp1 = w + (size_t)(r1 + min(ln, ROWS - 1)) * K + 8 * lg;
+  const bf16_t* wp2 = w + (size_t)(r2 + min(ln, ROWS - 1)) * K + 8 * lg;
   const bf16_t* xp = x + (size_t)min(ln, M - 1) * ldx + 8 * lg;
   gs_f32x4_t acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
 
@@ -281,8 +283,8 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     for (int u = 0; u < U; ++u) {
       const int kk = k + 32 * u;
       const bool ok = kk + 8 * lg < ke;
-      w1[u].u = ok ? *reinterpret_cast<const uint4*>(wp1 + kk) : make_uint4(0, 0, 0, 0);
-      w2[u].u = ok ? *reinterpret_cast<const uint4*>(wp2 + kk) : make_uint4(0, 0, 0, 0);
+      w1[u].u = (ok && wrow) ? *reinterpret_cast<const uint4*>(wp1 + kk) : make_uint4(0, 0, 0, 0);
+      w2[u].u = (ok && wrow) ? *reinterpret_cast<const uint4*>(wp2 + kk) : make_uint4(0, 0, 0, 0);
       xf[u].u = (ok && ln < M) ? *reinterpret_cast<const uint4*>(xp + kk) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
@@ -309,7 +311,7 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
       const int c = r1 + 4 * lg + i;
       // the gate and up products are rounded to bfloat16 as the unfused path stores them
       const float g = round_to<bf16_t>(acc1[i]), u = round_to<bf16_t>(acc2[i]);
-      if (c < N_out) y[(size_t)m * ldy + c] = float_to_bf16(g / (1.0f + expf(-g)) * u);
+      if (4 * lg + i < ROWS && c < N_out) y[(size_t)m * ldy + c] = float_to_bf16(g / (1.0f + expf(-g)) * u);
     }
   } else {
     const int D = rs.D, half = D >> 1;
@@ -328,7 +330,8 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     if (dst == nullptr) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int j = 16 * tile + 4 * lg + i;      // column in the first half of the head
+      if (4 * lg + i >= ROWS) continue;
+      const int j = ROWS * tile + 4 * lg + i;    // column in the first half of the head
       // as in the unfused path, the projection is rounded to bfloat16 before the rotation
       float x1 = round_to<bf16_t>(acc1[i]), x2 = round_to<bf16_t>(acc2[i]);
       if ((is_q || is_k) && rs.inv_freq) {
@@ -360,7 +363,7 @@ extern "C" int ptl_gate_up_silu_bf16(void* out, const void* x, const void* w, in
   const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
   RopeStoreArgs none = {};
-  gemm_pair_kernel<PAIR_SILU, 8><<<blocks, waves * 64, lds, stream>>>(
+  gemm_pair_kernel<PAIR_SILU, 8, 16><<<blocks, waves * 64, lds, stream>>>(
       (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, I, K, ldx, I, k_per_wave, I, blocks, 0, none);
   return ptl_launch_status();
 }
@@ -375,14 +378,21 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
   if (M > 16 || Hq <= 0 || Hkv <= 0 || D <= 0 || D % 32 || K <= 0 || K % 8 || ldx % 8 || ldx < K ||
       ldq < (long)Hq * D || page_size <= 0 || !positions || (slots && (!k_cache || !v_cache)))
     return PTL_ERR_ARG;
-  const int tiles = D / 32;                       // 16-wide tiles in half a head
+  // few heads: 8-column tiles, so that twice as many workgroups share the weight stream
+  const bool small = (Hq + 2 * Hkv) * (D / 32) <= 160;
+  const int tiles = small ? D / 16 : D / 32;      // tiles in half a head
   const int blocks = (Hq + 2 * Hkv) * tiles;
   const int waves = pair_waves(blocks, K);
   const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
   RopeStoreArgs rs = {positions, inv_freq, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, Hq, Hkv, D, page_size};
-  gemm_pair_kernel<PAIR_ROPE, 8><<<blocks, waves * 64, lds, stream>>>(
-      (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,
-      tiles, D, rs);
+  if (small)
+    gemm_pair_kernel<PAIR_ROPE, 8, 8><<<blocks, waves * 64, lds, stream>>>(
+        (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,
+        tiles, D, rs);
+  else
+    gemm_pair_kernel<PAIR_ROPE, 8, 16><<<blocks, waves * 64, lds, stream>>>(
+        (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,
+        tiles, D, rs);
   return ptl_launch_status();
 }
