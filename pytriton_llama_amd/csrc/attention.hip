@@ -19,6 +19,7 @@
 // ptl_attention_generic: vector-FMA kernel, float32 math, storage type T
 // (float32 or bfloat16), any page size, any D up to 256.
 #include "common.h"
+#include "mfma.h"
 #include <math.h>
 
 #define BM 16
@@ -461,325 +462,6 @@ extern "C" int ptl_attention_decode(void* out, long out_stride, const void* q, l
 }
 
 // ===========================================================================
-// ptl_attention_prefill_mfma: bfloat16 prompt portions on the matrix cores.
-//
-// A workgroup of four waves takes 64 or 128 query rows of one head (16 or 32 per
-// wave) and walks the sequence's keys in tiles of 64, through LDS; the next tile
-// is on its way from global memory while the current one is used. Both products are
-// computed transposed so that the scores leave the first MFMA in the register
-// layout the second one wants, without a shuffle:
-//   S^T[key, query] = K[key, :] . Q[query, :]      (A = K tile, B = Q^T)
-//   O^T[d, query]  += V^T[d, key] . P^T[key, query] (A = V^T tile, B = P^T)
-// with v_mfma_f32_16x16x32_bf16: a lane holds 8 consecutive k-values of row
-// (lane % 16), k-group (lane / 16); the result tile holds rows 4*(lane/16)+i,
-// column lane % 16. V^T is made when the value tile is written to LDS, with the
-// groups of four keys XOR-swizzled by the row so that reads and writes spread
-// over the banks. Softmax is the online one of
-// lite_llama/kernels/flashattentionv2.py:10-61 in base 2 (scale * log2 e folded
-// into the scores, exp2), float32 max / denominator / accumulator; P is rounded
-// to bfloat16 for the second product as there (:55).
-// Needs D % 32 == 0, D <= 128.
-// ===========================================================================
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-
-#define PF_BN 64
-
-union Frag8 {
-  uint4 u;
-  uint2 h[2];
-  bf16x8_t v;
-};
-
-// RT: 16-row query tiles per wave; the workgroup takes 64 * RT query rows.
-// (three workgroups a CU for head sizes up to 64: measured 1.4x faster than two at 8,192 keys)
-template <int NDT, int RT>
-__global__ void __launch_bounds__(256, NDT <= 2 ? 3 : 2)
-attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
-                         long q_stride, const bf16_t* __restrict__ k_cache,
-                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ q_start,
-                         const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ block_table,
-                         int bt_stride, const int32_t* __restrict__ work_seq,
-                         const int32_t* __restrict__ work_qoff, int Hq, int Hkv, int page_size,
-                         int page_shift, int window, float scale_log2) {
-  constexpr int D = 32 * NDT;
-  constexpr int PBM = 64 * RT;
-  constexpr int KS = D + 8;            // row stride of the key tile, in elements
-  constexpr int CPR = D / 8;           // 16-byte chunks per row
-  constexpr int NCH = PF_BN * CPR / 256;   // chunks of a tile per thread
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_BN * KS];
-  __shared__ __attribute__((aligned(16))) bf16_t Vt[D * PF_BN];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int ln = lane & 15, lg = lane >> 4;
-  const int head = blockIdx.y;
-  const int seq = work_seq[blockIdx.x];
-  const int qoff = work_qoff[blockIdx.x];
-  const int qs = q_start[seq];
-  const int qlen = q_start[seq + 1] - qs;
-  const int ctx = ctx_len[seq];
-  const int cached = ctx - qlen;
-  const int rows = min(PBM, qlen - qoff);
-  if (rows <= 0) return;
-  const int kvh = head / (Hq / Hkv);
-  const int32_t* bt = block_table + (size_t)seq * bt_stride;
-  const size_t page_elems = (size_t)Hkv * page_size * D;
-  const size_t kv_off = (size_t)kvh * page_size * D;
-  const int first_q = cached + qoff;
-
-  // query rows of this lane: tile r covers rows 16*(RT*wave + r) .. +15 of the block
-  int qpos[RT];
-  bool row_ok[RT];
-  Frag8 qf[RT][NDT];
-#pragma unroll
-  for (int r = 0; r < RT; ++r) {
-    const int my_row = 16 * (RT * wave + r) + ln;
-    row_ok[r] = my_row < rows;
-    const int qrow = row_ok[r] ? my_row : 0;       // rows past the end repeat row 0; never stored
-    qpos[r] = first_q + qrow;
-    const bf16_t* qp = q + (size_t)(qs + qoff + qrow) * q_stride + (size_t)head * D + 8 * lg;
-#pragma unroll
-    for (int kk = 0; kk < NDT; ++kk) qf[r][kk].u = *reinterpret_cast<const uint4*>(qp + 32 * kk);
-  }
-  const int wave_first_row = 16 * RT * wave;
-  const int wave_min_q = wave_first_row < rows ? first_q + wave_first_row : first_q;
-
-  f32x4_t o[RT][2 * NDT];
-  float m_run[RT], l_part[RT];
-#pragma unroll
-  for (int r = 0; r < RT; ++r) {
-    m_run[r] = -INFINITY;
-    l_part[r] = 0.f;
-#pragma unroll
-    for (int t = 0; t < 2 * NDT; ++t) o[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  }
-
-  const int k_end = min(ctx, first_q + rows);
-  const int k_lo = window > 0 ? max(0, first_q - window + 1) : 0;
-  const int k_begin = (k_lo / PF_BN) * PF_BN;
-
-  // registers that carry the next tile from global memory to LDS
-  uint4 kreg[NCH], vreg[NCH];
-  // page of a key position: a shift when the page size is a power of two
-  auto page_of = [&](int kp, int& off) -> int {
-    if (page_shift >= 0) { off = kp & (page_size - 1); return bt[kp >> page_shift]; }
-    const int pi = kp / page_size;
-    off = kp - pi * page_size;
-    return bt[pi];
-  };
-  auto fetch = [&](int k0) {
-    const bool full = k0 >= k_lo && k0 + PF_BN <= k_end;     // uniform: no per-key tests inside
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int c = tid + 256 * i;
-      const int r = c / CPR, cc = c - r * CPR;               // key tile: row r, chunk cc
-      const int key = c & (PF_BN - 1), dc = c / PF_BN;       // value tile: key, chunk dc
-      if (full) {
-        int off;
-        int page = page_of(k0 + r, off);
-        kreg[i] = *reinterpret_cast<const uint4*>(
-            k_cache + (size_t)page * page_elems + kv_off + (size_t)off * D + cc * 8);
-        page = page_of(k0 + key, off);
-        vreg[i] = *reinterpret_cast<const uint4*>(
-            v_cache + (size_t)page * page_elems + kv_off + (size_t)off * D + dc * 8);
-      } else {
-        kreg[i] = make_uint4(0, 0, 0, 0);
-        vreg[i] = make_uint4(0, 0, 0, 0);
-        int kp = k0 + r, off;
-        if (kp >= k_lo && kp < k_end) {
-          const int page = page_of(kp, off);
-          if (page >= 0)
-            kreg[i] = *reinterpret_cast<const uint4*>(
-                k_cache + (size_t)page * page_elems + kv_off + (size_t)off * D + cc * 8);
-        }
-        kp = k0 + key;
-        if (kp >= k_lo && kp < k_end) {
-          const int page = page_of(kp, off);
-          if (page >= 0)
-            vreg[i] = *reinterpret_cast<const uint4*>(
-                v_cache + (size_t)page * page_elems + kv_off + (size_t)off * D + dc * 8);
-        }
-      }
-    }
-  };
-  auto stash = [&]() {
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int c = tid + 256 * i;
-      {
-        const int r = c / CPR, cc = c - r * CPR;
-        *reinterpret_cast<uint4*>(Ks + r * KS + cc * 8) = kreg[i];
-      }
-      {
-        const int key = c & (PF_BN - 1), dc = c / PF_BN;
-        union { uint4 u; bf16_t e[8]; } val;
-        val.u = vreg[i];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int d = dc * 8 + j;
-          Vt[d * PF_BN + ((((key >> 2) ^ (d & 15)) << 2) | (key & 3))] = val.e[j];
-        }
-      }
-    }
-  };
-
-  fetch(k_begin);
-  for (int k0 = k_begin; k0 < k_end; k0 += PF_BN) {
-    __syncthreads();                    // everyone has left the previous tile
-    stash();
-    __syncthreads();                    // the tile is in LDS
-    if (k0 + PF_BN < k_end) fetch(k0 + PF_BN);     // the next tile travels while this one is used
-
-    // a wave whose rows all lie before this tile has nothing to do in it
-    const int wave_max_q = first_q + min(rows, wave_first_row + 16 * RT) - 1;
-    if (wave_first_row >= rows || k0 > wave_max_q) continue;
-
-    f32x4_t st[RT][4];
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-#pragma unroll
-      for (int r = 0; r < RT; ++r) st[r][kt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < NDT; ++kk) {
-        Frag8 a;
-        a.u = *reinterpret_cast<const uint4*>(Ks + (16 * kt + ln) * KS + 32 * kk + 8 * lg);
-#pragma unroll
-        for (int r = 0; r < RT; ++r)
-          st[r][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[r][kk].v, st[r][kt], 0, 0, 0);
-      }
-    }
-    // only tiles that touch the diagonal, the end of the keys or a window's edge need masks
-    const bool need_mask = (k0 + PF_BN - 1 > wave_min_q) || (k0 + PF_BN > k_end) || window > 0;
-    Frag8 pb[RT][2];
-#pragma unroll
-    for (int r = 0; r < RT; ++r) {
-      if (need_mask) {
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int key = k0 + 16 * kt + 4 * lg + i;
-            const bool vis = key <= qpos[r] && key < k_end && (window <= 0 || key > qpos[r] - window);
-            st[r][kt][i] = vis ? st[r][kt][i] : -INFINITY;
-          }
-      }
-      // the running max is kept in units of the raw scores; scale * log2(e) enters in the
-      // exponent's multiply-add
-      float tmax = -INFINITY;
-#pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
-        tmax = fmaxf(tmax, fmaxf(fmaxf(st[r][kt][0], st[r][kt][1]), fmaxf(st[r][kt][2], st[r][kt][3])));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m_run[r], tmax);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      if (__any(m_new > m_run[r])) {           // the max moved for some row: rescale what is kept
-        const float alpha = __builtin_amdgcn_exp2f((m_run[r] - m_safe) * scale_log2);
-        l_part[r] *= alpha;
-#pragma unroll
-        for (int t = 0; t < 2 * NDT; ++t) {
-          o[r][t][0] *= alpha; o[r][t][1] *= alpha; o[r][t][2] *= alpha; o[r][t][3] *= alpha;
-        }
-      }
-      m_run[r] = m_new;
-      const float mc = -m_safe * scale_log2;
-#pragma unroll
-      for (int half = 0; half < 2; ++half)
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float p = __builtin_amdgcn_exp2f(fmaf(st[r][2 * half + t][i], scale_log2, mc));
-            l_part[r] += p;
-            pb[r][half].v[4 * t + i] = (__bf16)p;
-          }
-    }
-#pragma unroll
-    for (int half = 0; half < 2; ++half)
-#pragma unroll
-      for (int dt = 0; dt < 2 * NDT; ++dt) {
-        const int d = 16 * dt + ln;
-        const int g0 = 8 * half + lg, g1 = g0 + 4;
-        Frag8 a;
-        a.h[0] = *reinterpret_cast<const uint2*>(Vt + d * PF_BN + ((g0 ^ ln) << 2));
-        a.h[1] = *reinterpret_cast<const uint2*>(Vt + d * PF_BN + ((g1 ^ ln) << 2));
-#pragma unroll
-        for (int r = 0; r < RT; ++r)
-          o[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb[r][half].v, o[r][dt], 0, 0, 0);
-      }
-  }
-
-#pragma unroll
-  for (int r = 0; r < RT; ++r) {
-    float l = l_part[r] + __shfl_xor(l_part[r], 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    if (row_ok[r]) {
-      const float inv = l > 0.f ? 1.0f / l : 0.f;
-      const int my_row = 16 * (RT * wave + r) + ln;
-      bf16_t* op = out + (size_t)(qs + qoff + my_row) * out_stride + (size_t)head * D + 4 * lg;
-#pragma unroll
-      for (int dt = 0; dt < 2 * NDT; ++dt) {
-        union { uint2 u; bf16_t e[4]; } rr;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) rr.e[i] = float_to_bf16(o[r][dt][i] * inv);
-        *reinterpret_cast<uint2*>(op + 16 * dt) = rr.u;
-      }
-    }
-  }
-}
-
-template <int NDT, int RT>
-static int launch_prefill_mfma(void* out, long out_stride, const void* q, long q_stride,
-                               const void* k_cache, const void* v_cache, const int32_t* q_start,
-                               const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
-                               const int32_t* work_seq, const int32_t* work_qoff, int n_work, int Hq,
-                               int Hkv, int page_size, int window, float scale, hipStream_t stream) {
-  dim3 grid(n_work, Hq);
-  int page_shift = -1;
-  for (int sh = 0; sh < 31; ++sh)
-    if ((1 << sh) == page_size) page_shift = sh;
-  attn_prefill_mfma_kernel<NDT, RT><<<grid, 256, 0, stream>>>(
-      (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-      (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff, Hq, Hkv,
-      page_size, page_shift, window, scale * 1.4426950408889634f);
-  return ptl_launch_status();
-}
-
-// work_seq / work_qoff list query blocks of ``block_rows`` rows (64 or 128). bfloat16 only;
-// q rows must be 16-byte aligned and output rows 8-byte (q_stride % 8, out_stride % 4).
-extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void* q, long q_stride,
-                                          const void* k_cache, const void* v_cache,
-                                          const int32_t* q_start, const int32_t* ctx_len,
-                                          const int32_t* block_table, int bt_stride,
-                                          const int32_t* work_seq, const int32_t* work_qoff,
-                                          int n_work, int block_rows, int Hq, int Hkv, int D,
-                                          int page_size, int window, float scale,
-                                          hipStream_t stream) {
-  if (n_work <= 0) return PTL_OK;
-  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D % 32 || D <= 0 || D > 128 || page_size <= 0 ||
-      Hq > 65535 || q_stride % 8 || out_stride % 4 || (block_rows != 64 && block_rows != 128))
-    return PTL_ERR_ARG;
-#define GO(N, R) launch_prefill_mfma<N, R>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
-                                           ctx_len, block_table, bt_stride, work_seq, work_qoff,  \
-                                           n_work, Hq, Hkv, page_size, window, scale, stream)
-  if (block_rows == 64) {
-    switch (D / 32) {
-      case 1: return GO(1, 1);
-      case 2: return GO(2, 1);
-      case 3: return GO(3, 1);
-      default: return GO(4, 1);
-    }
-  }
-  switch (D / 32) {
-    case 1: return GO(1, 2);
-    case 2: return GO(2, 2);
-    case 3: return GO(3, 2);
-    default: return GO(4, 2);
-  }
-#undef GO
-}
-
-// ===========================================================================
 // ptl_attention_decode_mfma: the bfloat16 decode case on the matrix cores.
 //
 // Same grid and split scheme as ptl_attention_decode, but a wave takes 16 keys
@@ -795,7 +477,6 @@ extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void
 // that head's column; the four waves and the splits are merged at the end as
 // in ptl_attention_decode. Needs D % 32 == 0, D <= 128, Hq/Hkv <= 16.
 // ===========================================================================
-typedef short s16x4_t __attribute__((ext_vector_type(4)));
 // 16-key tiles a wave has in flight per turn; measured on MI355X: 2 beats 4 (more
 // workgroups fit a CU) and 1 (more turns) from head size 64 to 128
 #ifndef DEC_UNR

@@ -390,6 +390,15 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         "attention_decode")
 
 
+def attention_prefill_mfma_fits(dtype: torch.dtype, num_kv_heads: int, head_dim: int,
+                                page_size: int) -> bool:
+    """Whether ``attention_prefill_mfma`` takes this case: bfloat16, head size 32, 64, 96 or
+    128, a page size that is a power of two, pages (of all kv heads) below 4 GiB."""
+    return (dtype == torch.bfloat16 and head_dim % 32 == 0 and 0 < head_dim <= 128
+            and page_size > 0 and page_size & (page_size - 1) == 0
+            and num_kv_heads * page_size * head_dim * 2 < 2 ** 32)
+
+
 def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                            v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                            block_table: torch.Tensor, work_seq: torch.Tensor,
@@ -403,6 +412,9 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
         raise KernelError("attention_prefill_mfma: bfloat16 only")
     if D % 32 or D > 128:
         raise KernelError(f"attention_prefill_mfma: head size {D} is not 32, 64, 96 or 128")
+    if not attention_prefill_mfma_fits(q.dtype, Hkv, D, page_size):
+        raise KernelError(f"attention_prefill_mfma: page size {page_size} is not a power of two "
+                          "(or a page of all kv heads reaches 4 GiB)")
     _need_gpu(work_seq, work_qoff)
     _i32(work_seq, "work_seq")
     _i32(work_qoff, "work_qoff")
@@ -412,7 +424,7 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
         raise KernelError("attention_prefill_mfma: query blocks are 64 or 128 rows")
     if q.stride(0) % 8 or out.stride(0) % 4 or q.data_ptr() % 16 or out.data_ptr() % 8:
         raise KernelError("attention_prefill_mfma: q rows must be 16-byte aligned, out rows 8-byte")
-    lib = library.load("attention")
+    lib = library.load("attention_prefill")
     _check(lib.ptl_attention_prefill_mfma(
         _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
         _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),

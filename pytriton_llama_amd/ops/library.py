@@ -25,7 +25,11 @@ ARCH = "gfx950"
 HIPCC_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-shared", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
-KERNEL_LIBRARIES = ("embedding", "norm", "rope", "attention", "activation", "gemm", "sampling")
+KERNEL_LIBRARIES = ("embedding", "norm", "rope", "attention", "attention_prefill", "activation",
+                    "gemm", "sampling")
+# options of single sources. attention_prefill: no value there is a NaN unless an input is, and
+# without the promise every maximum of scores is preceded by instructions that quiet its inputs
+EXTRA_FLAGS = {"attention_prefill": ["-fno-honor-nans"]}
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -89,7 +93,8 @@ def is_stale(name: str) -> bool:
 
 
 def compile_command(name: str, out: str) -> List[str]:
-    return [_hipcc()] + HIPCC_FLAGS + ["-I", CSRC_DIR, "-o", out, source_path(name)]
+    return ([_hipcc()] + HIPCC_FLAGS + EXTRA_FLAGS.get(name, []) +
+            ["-I", CSRC_DIR, "-o", out, source_path(name)])
 
 
 def build(names: Iterable[str] = KERNEL_LIBRARIES, force: bool = False, verbose: bool = True) -> None:

@@ -45,6 +45,8 @@ class PagedAttention(Part):
         self.qkv: Optional[torch.Tensor] = None
         self.o: Optional[torch.Tensor] = None
         libs = ("attention", "rope") + LINEAR_LIBRARIES
+        if self.head_dim % 32 == 0 and self.head_dim <= 128:
+            libs += ("attention_prefill",)          # the matrix-core kernel for prompt portions
         if position is not None:
             libs += tuple(position.kernel_libraries)
         self.kernel_libraries = tuple(dict.fromkeys(libs))
@@ -130,7 +132,8 @@ class PagedAttention(Part):
                                  self.decode_splits(ctx, n_dec, mfma), matrix_cores=mfma)
         if n_dec == ctx.num_seqs:
             return
-        if q.dtype == torch.bfloat16 and D % 32 == 0 and D <= 128:
+        if (ops.attention_prefill_mfma_fits(q.dtype, self.num_kv_heads, D, cache.page_size)
+                and q.stride(0) % 8 == 0):
             # long portions in 128-row blocks (keys and values are staged half as often)
             rows = 128 if ctx.max_q_len >= 256 else 64
             ws, wo = ctx.work["multi128" if rows == 128 else "multi64"]

@@ -323,8 +323,9 @@ def test_attention_decode_window(ops, dtype):
 @pytest.mark.parametrize("case", [
     dict(seq_lens=[40], q_lens=[40], Hq=4, Hkv=4, D=64, P=16),
     dict(seq_lens=[200, 64, 33], q_lens=[130, 2, 33], Hq=6, Hkv=1, D=128, P=8),
-    dict(seq_lens=[150], q_lens=[70], Hq=2, Hkv=1, D=32, P=5),
+    dict(seq_lens=[150], q_lens=[70], Hq=2, Hkv=1, D=32, P=32),
     dict(seq_lens=[129, 300], q_lens=[129, 65], Hq=4, Hkv=2, D=96, P=16),
+    dict(seq_lens=[450], q_lens=[333], Hq=2, Hkv=1, D=64, P=128),      # a page longer than a tile
     dict(seq_lens=[1, 2, 64, 65], q_lens=[1, 2, 64, 65], Hq=2, Hkv=2, D=64, P=4),
 ])
 @pytest.mark.parametrize("kernel", ["mfma", "mfma128"])
@@ -336,6 +337,15 @@ def test_attention_prefill_mfma(ops, case, kernel):
 def test_attention_prefill_mfma_window(ops, kernel):
     _attention_case(ops, torch.bfloat16, seq_lens=[300, 90], q_lens=[150, 25], Hq=4, Hkv=2, D=64,
                     P=8, window=70, kernel=kernel)
+
+
+def test_attention_prefill_mfma_refuses_odd_page_size(ops):
+    """A page size that is no power of two is for the general kernel; the fast one says so."""
+    assert not ops.attention_prefill_mfma_fits(torch.bfloat16, 1, 32, 5)
+    assert ops.attention_prefill_mfma_fits(torch.bfloat16, 1, 32, 8)
+    with pytest.raises(ops.KernelError, match="power of two"):
+        _attention_case(ops, torch.bfloat16, seq_lens=[150], q_lens=[70], Hq=2, Hkv=1, D=32, P=5,
+                        kernel="mfma")
 
 
 def test_attention_prefill_mfma_long(ops):
