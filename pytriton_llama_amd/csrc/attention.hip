@@ -464,37 +464,52 @@ extern "C" int ptl_attention_decode(void* out, long out_stride, const void* q, l
 // ===========================================================================
 // ptl_attention_decode_mfma: the bfloat16 decode case on the matrix cores.
 //
-// Same grid and split scheme as ptl_attention_decode, but a wave takes 16 keys
-// per turn and all query heads of a kv head at once (up to 16 of them are the N
-// side of the MFMA tiles, so grouped heads cost nothing extra):
+// Same grid and split scheme as ptl_attention_decode, but a wave takes UNR tiles of
+// 16 keys per turn and all query heads of a kv head at once (up to 16 of them are
+// the N side of the MFMA tiles, so grouped heads cost nothing extra):
 //   S^T[key, head] = K[key, :] . Q[head, :]         v_mfma_f32_16x16x32_bf16,
 //                                                   A = 16-byte loads of key rows
 //   O^T[d, head]  += V^T[d, key] . P^T[key, head]   v_mfma_f32_16x16x16_bf16,
 //                                                   B = P^T as it leaves the
-//                                                   first product, A = values
-//                                                   gathered by (d, key)
+//                                                   first product, A = V^T
+// The value tiles go through a region of LDS that belongs to the wave: written as
+// they lie in the cache (rows of D, 16-byte stores), read back transposed with
+// ds_read_b64_tr_b16 (in a group of 16 lanes, lane s points at
+// V[4 g + s/4][16 t + 4 (s%4)] and lane l receives V[4 g + 0..3][16 t + l]).
+// Nothing in the loop waits for another wave. The keys and values of the next turn
+// are on their way from global memory while this turn is computed, and the page
+// numbers of the turn after that are read one turn earlier still.
 // The softmax state of a head (running max, denominator) lives in the lanes of
 // that head's column; the four waves and the splits are merged at the end as
-// in ptl_attention_decode. Needs D % 32 == 0, D <= 128, Hq/Hkv <= 16.
+// in ptl_attention_decode. Needs D % 32 == 0, D <= 128, Hq/Hkv <= 16, a page size
+// that is a power of two, pages (of all kv heads) below 4 GiB.
 // ===========================================================================
-// 16-key tiles a wave has in flight per turn; measured on MI355X: 2 beats 4 (more
-// workgroups fit a CU) and 1 (more turns) from head size 64 to 128
-#ifndef DEC_UNR
-#define DEC_UNR(NDT) 2
-#endif
+__device__ __forceinline__ void wave_lds_fence() {
+  // orders this wave's LDS writes and reads for the compiler; the LDS itself runs a wave's
+  // instructions in order
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
-template <int NDT>
+template <int NDT, int UNR>
 __global__ void __launch_bounds__(256)
 attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q,
                         long q_stride, const bf16_t* __restrict__ k_cache,
                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ q_start,
                         const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ block_table,
                         int bt_stride, float* __restrict__ part_acc, float* __restrict__ part_ml,
-                        int Hq, int Hkv, int page_size, int window, float scale_log2, int num_splits) {
+                        int Hq, int Hkv, int page_size, int page_shift, int window, float scale_log2,
+                        int num_splits) {
   constexpr int D = 32 * NDT;
   constexpr int NT = 2 * NDT;             // 16-wide tiles of the head dimension
+  constexpr int TILE = 64 * UNR;          // keys per turn of the workgroup
+  constexpr int VS = D + 16;              // row stride of a value tile in LDS, in elements
+  constexpr int CPR = D / 8;              // 16-byte chunks per row
+  constexpr int VCH = 16 * CPR / 64;      // chunks of a tile per lane
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 15, lg = lane >> 4;
+  const int xor16 = 4 * (lane ^ 16), xor32 = 4 * (lane ^ 32);
   const int seq = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int G = Hq / Hkv;
   const int head0 = kvh * G;
@@ -502,14 +517,15 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
   const int ctx = ctx_len[seq];
   const int k_lo = window > 0 ? max(0, ctx - window) : 0;
   const int span = ctx - k_lo;
-  constexpr int UNR = DEC_UNR(NDT);       // 16-key tiles a wave loads ahead
-  constexpr int TILE = 64 * UNR;          // keys per turn of the workgroup
   const int per_split = ((span + num_splits - 1) / num_splits + TILE - 1) / TILE * TILE;
   const int k_begin = k_lo + split * per_split;
   const int k_end = min(ctx, k_begin + per_split);
+  const int turns = (k_end - k_begin + TILE - 1) / TILE;
   const int32_t* bt = block_table + (size_t)seq * bt_stride;
-  const size_t head_pages = (size_t)Hkv * page_size * D;     // elements per page
-  const size_t kv_off = (size_t)kvh * page_size * D;
+  const uint32_t page_bytes = (uint32_t)Hkv * page_size * D * 2;
+  const int page_mask = page_size - 1;
+  const char* k_head = reinterpret_cast<const char*>(k_cache) + (size_t)kvh * page_size * D * 2;
+  const char* v_head = reinterpret_cast<const char*>(v_cache) + (size_t)kvh * page_size * D * 2;
 
   Frag8 qf[NDT];
 #pragma unroll
@@ -524,98 +540,126 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
   for (int t = 0; t < NT; ++t) o[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_part = 0.f;
 
-  // values go through LDS: each wave copies its tiles row by row (coalesced 16-byte
-  // loads) into a region of its own and reads them back by (d, key) for the second product
-  constexpr int VS = D + 4;               // row stride in elements: rows 4 apart fall 8 banks apart
-  constexpr int CPR = D / 8;              // 16-byte chunks per row
-  constexpr int VCH = 16 * CPR / 64;      // chunks of a tile per lane
   extern __shared__ float lds[];
   bf16_t* vl = reinterpret_cast<bf16_t*>(lds) + (size_t)wave * UNR * 16 * VS;
-  const int turns = (k_end - k_begin + TILE - 1) / TILE;
-  for (int turn = 0; turn < turns; ++turn) {
-    const int kc = k_begin + turn * TILE + 16 * UNR * wave;
-    Frag8 kf[UNR][NDT];
-    uint4 vg[UNR][VCH];
+  // this lane's chunks of a value tile: row vrow[i], elements vcol[i] .. +7
+  int vrow[VCH], vcol[VCH];
+#pragma unroll
+  for (int i = 0; i < VCH; ++i) {
+    const int c = lane + 64 * i;
+    vrow[i] = c / CPR;
+    vcol[i] = (c - vrow[i] * CPR) * 8;
+  }
+
+  int pk[UNR], pv[UNR][VCH];            // pages of the key row and of the value chunks' rows
+  uint4 vg[UNR][VCH];                   // values on their way to LDS
+  auto first_key = [&](int turn) { return k_begin + turn * TILE + 16 * UNR * wave; };
+  auto load_pages = [&](int turn) {
+    const int kc = first_key(turn);
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int kb = kc + 16 * u;
-      {
-        const int kp = kb + ln;                   // row ln of the key tile (first product)
-        const bool ok = kp < k_end;
-        const bf16_t* kr = k_cache;
-        if (ok) {
-          const int page = bt[kp / page_size];
-          kr = k_cache + (size_t)page * head_pages + kv_off + (size_t)(kp % page_size) * D + 8 * lg;
-        }
-#pragma unroll
-        for (int kk = 0; kk < NDT; ++kk)
-          kf[u][kk].u = ok ? *reinterpret_cast<const uint4*>(kr + 32 * kk) : make_uint4(0, 0, 0, 0);
-      }
+      const int kp = kc + 16 * u + ln;
+      pk[u] = (turn < turns && kp < k_end) ? bt[kp >> page_shift] : -1;
 #pragma unroll
       for (int i = 0; i < VCH; ++i) {
-        const int c = lane + 64 * i;
-        const int kp = kb + c / CPR;
-        vg[u][i] = make_uint4(0, 0, 0, 0);
-        if (kp < k_end) {
-          const int page = bt[kp / page_size];
-          vg[u][i] = *reinterpret_cast<const uint4*>(
-              v_cache + (size_t)page * head_pages + kv_off + (size_t)(kp % page_size) * D + (c % CPR) * 8);
-        }
+        const int vp = kc + 16 * u + vrow[i];
+        pv[u][i] = (turn < turns && vp < k_end) ? bt[vp >> page_shift] : -1;
       }
     }
-#pragma unroll
-    for (int u = 0; u < UNR; ++u)
-#pragma unroll
-      for (int i = 0; i < VCH; ++i) {
-        const int c = lane + 64 * i;
-        uint2* dst = reinterpret_cast<uint2*>(vl + (size_t)(u * 16 + c / CPR) * VS + (c % CPR) * 8);
-        dst[0] = make_uint2(vg[u][i].x, vg[u][i].y);
-        dst[1] = make_uint2(vg[u][i].z, vg[u][i].w);
-      }
-    __syncthreads();
-    s16x4_t vf[UNR][NT];
-#pragma unroll
-    for (int u = 0; u < UNR; ++u)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-          vf[u][t][j] = (short)vl[(size_t)(u * 16 + 4 * lg + j) * VS + 16 * t + ln];
+  };
+  auto issue_loads = [&](int turn, Frag8 (&kf)[UNR][NDT]) {
+    const int kc = first_key(turn);
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int kb = kc + 16 * u;
-      if (kb >= k_end) break;                     // wave-uniform
-      f32x4_t st = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const int kp = kc + 16 * u + ln;
+      const char* kr = k_head + (size_t)(uint32_t)max(pk[u], 0) * page_bytes +
+                       (uint32_t)(((kp & page_mask) * D + 8 * lg) * 2);
 #pragma unroll
       for (int kk = 0; kk < NDT; ++kk)
-        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][kk].v, qf[kk].v, st, 0, 0, 0);
-      float tmax = -INFINITY;
+        kf[u][kk].u = pk[u] >= 0 ? *reinterpret_cast<const uint4*>(kr + 64 * kk) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < VCH; ++i) {
+        const int vp = kc + 16 * u + vrow[i];
+        vg[u][i] = make_uint4(0, 0, 0, 0);              // rows past the end read as zeros
+        if (pv[u][i] >= 0)
+          vg[u][i] = *reinterpret_cast<const uint4*>(
+              v_head + (size_t)(uint32_t)pv[u][i] * page_bytes +
+              (uint32_t)(((vp & page_mask) * D + vcol[i]) * 2));
+      }
+    }
+  };
+  // one turn: the values that arrived go to LDS, the next turn's loads are issued, this
+  // turn's keys (in kf) and values (in LDS) are used
+  auto step = [&](int turn, Frag8 (&kf)[UNR][NDT], Frag8 (&kf_next)[UNR][NDT]) {
+    wave_lds_fence();                                   // the last turn's reads are done
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+#pragma unroll
+      for (int i = 0; i < VCH; ++i)
+        *reinterpret_cast<uint4*>(vl + (u * 16 + vrow[i]) * VS + vcol[i]) = vg[u][i];
+    wave_lds_fence();
+    if (turn + 1 < turns) {
+      issue_loads(turn + 1, kf_next);
+      load_pages(turn + 2);
+    }
+    const int kc = first_key(turn);
+    if (kc >= k_end) return;                            // wave-uniform: nothing of this turn is ours
+    f32x4_t st[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      st[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NDT; ++kk)
+        st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][kk].v, qf[kk].v, st[u], 0, 0, 0);
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float s = st[i] * scale_log2;
-        s = (kb + 4 * lg + i < k_end) ? s : -INFINITY;
-        st[i] = s;
-        tmax = fmaxf(tmax, s);
+        float sc = st[u][i] * scale_log2;
+        sc = (kc + 16 * u + 4 * lg + i < k_end) ? sc : -INFINITY;
+        st[u][i] = sc;
+        tmax = fmaxf(tmax, sc);
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m_run, tmax);      // finite: key kb is in range
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-      m_run = m_new;
+    tmax = fmaxf(tmax, __int_as_float(__builtin_amdgcn_ds_bpermute(xor16, __float_as_int(tmax))));
+    tmax = fmaxf(tmax, __int_as_float(__builtin_amdgcn_ds_bpermute(xor32, __float_as_int(tmax))));
+    if (tmax > m_run) {                                 // (finite: key kc is in range)
+      const float alpha = __builtin_amdgcn_exp2f(m_run - tmax);
+      m_run = tmax;
       l_part *= alpha;
-      s16x4_t pb;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = __builtin_amdgcn_exp2f(st[i] - m_new);
-        l_part += p;
-        pb[i] = (short)float_to_bf16(p);
-      }
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         o[t][0] *= alpha; o[t][1] *= alpha; o[t][2] *= alpha; o[t][3] *= alpha;
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[u][t], pb, o[t], 0, 0, 0);
       }
     }
+    s16x4_t pb[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __builtin_amdgcn_exp2f(st[u][i] - m_run);
+        l_part += p;
+        pb[u][i] = (short)float_to_bf16(p);
+      }
+    const bf16_t* vp = vl + (4 * lg + (ln >> 2)) * VS + 4 * (ln & 3);
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const s16x4_t vf = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4_t*)(vp + u * 16 * VS + 16 * t));
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pb[u], o[t], 0, 0, 0);
+      }
+  };
+
+  Frag8 kfa[UNR][NDT], kfb[UNR][NDT];
+  load_pages(0);
+  issue_loads(0, kfa);
+  load_pages(1);
+  for (int turn = 0; turn < turns; turn += 2) {
+    step(turn, kfa, kfb);
+    if (turn + 1 < turns) step(turn + 1, kfb, kfa);
   }
 
   float l = l_part + __shfl_xor(l_part, 16, 64);
@@ -657,7 +701,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
   }
 }
 
-template <int NDT>
+template <int NDT, int UNR>
 static int launch_decode_mfma(void* out, long out_stride, const void* q, long q_stride,
                               const void* k_cache, const void* v_cache, const int32_t* q_start,
                               const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
@@ -665,15 +709,16 @@ static int launch_decode_mfma(void* out, long out_stride, const void* q, long q_
                               int page_size, int window, float scale, int num_splits,
                               hipStream_t stream) {
   constexpr int D = 32 * NDT;
-  constexpr int UNR = DEC_UNR(NDT);
   dim3 grid(n_seq, Hkv, num_splits);
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
   const size_t lds_merge = (size_t)(4 * 16 * D + 4 * 16 * 2) * sizeof(float);
-  const size_t lds_values = (size_t)4 * UNR * 16 * (D + 4) * sizeof(bf16_t);
+  const size_t lds_values = (size_t)4 * UNR * 16 * (D + 16) * sizeof(bf16_t);
   const size_t lds = lds_merge > lds_values ? lds_merge : lds_values;
-  attn_decode_mfma_kernel<NDT><<<grid, 256, lds, stream>>>(
+  attn_decode_mfma_kernel<NDT, UNR><<<grid, 256, lds, stream>>>(
       (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
       (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, part_acc, part_ml, Hq, Hkv,
-      page_size, window, scale * 1.4426950408889634f, num_splits);
+      page_size, page_shift, window, scale * 1.4426950408889634f, num_splits);
   if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
   if (num_splits > 1) {
     dim3 mgrid(n_seq, Hq);
@@ -683,26 +728,37 @@ static int launch_decode_mfma(void* out, long out_stride, const void* q, long q_
   return ptl_launch_status();
 }
 
+// unroll: 16-key tiles a wave takes per turn, 1 or 2 (0: the kernel's choice).
 extern "C" int ptl_attention_decode_mfma(void* out, long out_stride, const void* q, long q_stride,
                                          const void* k_cache, const void* v_cache,
                                          const int32_t* q_start, const int32_t* ctx_len,
                                          const int32_t* block_table, int bt_stride, float* part_acc,
                                          float* part_ml, int n_seq, int Hq, int Hkv, int D,
                                          int page_size, int window, float scale, int num_splits,
-                                         hipStream_t stream) {
+                                         int unroll, hipStream_t stream) {
   if (n_seq <= 0) return PTL_OK;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hq / Hkv > 16 || D <= 0 || D % 32 || D > 128 ||
-      page_size <= 0 || q_stride % 8 || num_splits < 1 || num_splits > 1024 ||
-      (num_splits > 1 && (!part_acc || !part_ml)))
+      page_size <= 0 || (page_size & (page_size - 1)) ||
+      (long)Hkv * page_size * D * 2 >= (1L << 32) || q_stride % 8 || num_splits < 1 ||
+      num_splits > 1024 || (num_splits > 1 && (!part_acc || !part_ml)) || unroll < 0 || unroll > 2)
     return PTL_ERR_ARG;
-#define GO(N) launch_decode_mfma<N>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, ctx_len, \
-                                    block_table, bt_stride, part_acc, part_ml, n_seq, Hq, Hkv,      \
-                                    page_size, window, scale, num_splits, stream)
+  if (unroll == 0) unroll = 2;
+#define GO(N, U) launch_decode_mfma<N, U>(out, out_stride, q, q_stride, k_cache, v_cache, q_start,    \
+                                          ctx_len, block_table, bt_stride, part_acc, part_ml, n_seq, \
+                                          Hq, Hkv, page_size, window, scale, num_splits, stream)
+  if (unroll == 1) {
+    switch (D / 32) {
+      case 1: return GO(1, 1);
+      case 2: return GO(2, 1);
+      case 3: return GO(3, 1);
+      default: return GO(4, 1);
+    }
+  }
   switch (D / 32) {
-    case 1: return GO(1);
-    case 2: return GO(2);
-    case 3: return GO(3);
-    default: return GO(4);
+    case 1: return GO(1, 2);
+    case 2: return GO(2, 2);
+    case 3: return GO(3, 2);
+    default: return GO(4, 2);
   }
 #undef GO
 }

@@ -346,18 +346,25 @@ def _attention_common(out, q, k_cache, v_cache, q_start, ctx_len, block_table, w
     return T, Hq, Hkv, D, page_size
 
 
-def attention_decode_mfma_fits(dtype, Hq: int, Hkv: int, D: int) -> bool:
-    return dtype == torch.bfloat16 and D % 32 == 0 and D <= 128 and Hq // Hkv <= 16
+def attention_decode_mfma_fits(dtype, Hq: int, Hkv: int, D: int, page_size: int = 16) -> bool:
+    """Whether the matrix-core decode kernel takes this case: bfloat16, head size 32, 64, 96
+    or 128, at most 16 heads a kv head, a page size that is a power of two, pages (of all kv
+    heads) below 4 GiB."""
+    return (dtype == torch.bfloat16 and D % 32 == 0 and 0 < D <= 128 and Hq // Hkv <= 16
+            and page_size > 0 and page_size & (page_size - 1) == 0
+            and Hkv * page_size * D * 2 < 2 ** 32)
 
 
 def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                      v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                      block_table: torch.Tensor, n_seq: int, scale: float, window: int = 0,
-                     num_splits: int = 1, matrix_cores: bool = False) -> None:
+                     num_splits: int = 1, matrix_cores: bool = False, unroll: int = 0) -> None:
     """Split-KV attention of the first ``n_seq`` sequences of the tables, each of
     which brings exactly one query token (see csrc/attention.hip). Head sizes in
     steps of 16 up to 256, float32 or bfloat16. ``matrix_cores``: the MFMA
-    variant (bfloat16, head sizes 32/64/96/128, at most 16 heads a kv head)."""
+    variant (bfloat16, head sizes 32/64/96/128, at most 16 heads a kv head, a page
+    size that is a power of two); ``unroll``: its 16-key tiles per wave and turn
+    (1 or 2; 0 leaves the choice to the kernel)."""
     T, Hq, Hkv, D, page_size = _attention_common(out, q, k_cache, v_cache, q_start, ctx_len,
                                                  block_table, "attention_decode")
     if D % 16 or D > 256:
@@ -372,14 +379,16 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         part_ml = torch.empty((n_seq, Hq, num_splits, 2), dtype=torch.float32, device=q.device)
     lib = library.load("attention")
     if matrix_cores:
-        if not attention_decode_mfma_fits(q.dtype, Hq, Hkv, D) or q.stride(0) % 8 or q.data_ptr() % 16:
+        if (not attention_decode_mfma_fits(q.dtype, Hq, Hkv, D, page_size) or q.stride(0) % 8
+                or q.data_ptr() % 16):
             raise KernelError("attention_decode: the matrix-core variant needs bfloat16, a head "
-                              "size of 32/64/96/128, at most 16 heads a kv head, aligned q rows")
+                              "size of 32/64/96/128, at most 16 heads a kv head, a page size that "
+                              "is a power of two, aligned q rows")
         _check(lib.ptl_attention_decode_mfma(
             _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
             _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
             int(block_table.stride(0)), _ptr(part_acc), _ptr(part_ml), int(n_seq), Hq, Hkv, D,
-            page_size, int(window), ctypes.c_float(scale), int(num_splits), _stream()),
+            page_size, int(window), ctypes.c_float(scale), int(num_splits), int(unroll), _stream()),
             "attention_decode_mfma")
         return
     _check(lib.ptl_attention_decode(

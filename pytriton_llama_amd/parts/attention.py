@@ -118,14 +118,22 @@ class PagedAttention(Part):
         span = max(ctx.ctx_lens[:n_dec])
         if self.window:
             span = min(span, self.window)
-        want = -(-1024 // max(1, n_dec * groups))       # about a thousand workgroups (measured)
+        # measured on MI355X: the matrix-core kernel is best with about 512 workgroups (one
+        # round over the 256 CUs) and without splits once the batch brings half of that; the
+        # other one with about a thousand
+        base = max(1, n_dec * groups)
+        if matrix_cores:
+            want = 1 if base >= 256 else -(-512 // base)
+        else:
+            want = -(-1024 // base)
         return max(1, min(want, -(-span // turn), 64))
 
     def attend(self, out, q, cache, ctx, group) -> None:
         D, window = self.head_dim, self.window or 0
         n_dec = ctx.num_decode_seqs if D % 16 == 0 else 0
         if n_dec:
-            mfma = (ops.attention_decode_mfma_fits(q.dtype, self.num_heads, self.num_kv_heads, D)
+            mfma = (ops.attention_decode_mfma_fits(q.dtype, self.num_heads, self.num_kv_heads, D,
+                                                   cache.page_size)
                     and q.stride(0) % 8 == 0)
             ops.attention_decode(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
                                  group.block_table, n_dec, self.scale, window,
@@ -135,7 +143,7 @@ class PagedAttention(Part):
         if (ops.attention_prefill_mfma_fits(q.dtype, self.num_kv_heads, D, cache.page_size)
                 and q.stride(0) % 8 == 0):
             # long portions in 128-row blocks (keys and values are staged half as often)
-            rows = 128 if ctx.max_q_len >= 256 else 64
+            rows = 128 if ctx.max_q_len >= 256 and D <= 64 else 64
             ws, wo = ctx.work["multi128" if rows == 128 else "multi64"]
             ops.attention_prefill_mfma(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
                                        group.block_table, ws, wo, self.scale, window, rows)

@@ -225,7 +225,7 @@ def _paged_setup(seq_lens, q_lens, Hkv, D, P, dtype, seed, shuffle=True):
 
 
 def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=0, boost=None,
-                    kernel="generic", splits=1):
+                    kernel="generic", splits=1, unroll=0):
     kc, vc, bt, dk, dv = _paged_setup(seq_lens, q_lens, Hkv, D, P, dtype, seed)
     g = torch.Generator().manual_seed(seed + 100)
     T = sum(q_lens)
@@ -259,7 +259,7 @@ def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=
         assert all(ql == 1 for ql in q_lens)
         ops.attention_decode(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
                              bt.to(dev), len(q_lens), scale, window, splits,
-                             matrix_cores=(kernel == "decode_mfma"))
+                             matrix_cores=(kernel == "decode_mfma"), unroll=unroll)
     # plain: full causal attention over the sequence, rows of the portion kept
     for i, (s, ql) in enumerate(zip(seq_lens, q_lens)):
         full_q = torch.zeros(s, Hq, D)
@@ -302,11 +302,22 @@ def test_attention_decode(ops, dtype, splits, case):
     dict(seq_lens=[300, 64, 65, 1], Hq=4, Hkv=4, D=64, P=16),
     dict(seq_lens=[100, 257], Hq=32, Hkv=2, D=32, P=8),             # 16 heads a kv head
     dict(seq_lens=[90, 33, 700], Hq=3, Hkv=1, D=128, P=16),
-    dict(seq_lens=[70, 130], Hq=8, Hkv=2, D=96, P=5),               # odd page size
+    dict(seq_lens=[70, 130], Hq=8, Hkv=2, D=96, P=4),
+    dict(seq_lens=[500, 3, 129], Hq=4, Hkv=1, D=64, P=64),          # a page longer than a turn
 ])
-def test_attention_decode_mfma(ops, splits, case):
+@pytest.mark.parametrize("unroll", [1, 2])
+def test_attention_decode_mfma(ops, splits, case, unroll):
     _attention_case(ops, torch.bfloat16, q_lens=[1] * len(case["seq_lens"]), kernel="decode_mfma",
-                    splits=splits, **case)
+                    splits=splits, unroll=unroll, **case)
+
+
+def test_attention_decode_mfma_refuses_odd_page_size(ops):
+    """A page size that is no power of two is for the general kernel; the fast one says so."""
+    assert not ops.attention_decode_mfma_fits(torch.bfloat16, 8, 2, 96, 5)
+    assert ops.attention_decode_mfma_fits(torch.bfloat16, 8, 2, 96, 4)
+    with pytest.raises(ops.KernelError, match="power of two"):
+        _attention_case(ops, torch.bfloat16, seq_lens=[70, 130], q_lens=[1, 1], Hq=8, Hkv=2, D=96,
+                        P=5, kernel="decode_mfma")
 
 
 def test_attention_decode_mfma_window(ops):
