@@ -116,12 +116,26 @@ union GsFrag {
   gs_bf16x8_t v;
 };
 
+// The follow-up of a product whose result is added to the residual stream and normalised
+// (ptl_gemm_skinny_add_norm_bf16). The normalisation needs the whole row, which no workgroup
+// has, so the product's kernel does what it can see: s = round_bf16(x W^T) + residual, the
+// sum written back as the new residual, y = bf16(s * norm_w) and the sum of s^2 over the
+// workgroup's columns into partials[m][workgroup]. The kernel that consumes y multiplies its
+// own results by rsqrt(mean(s^2) + eps), which it gets from the partials (RowScaleArgs).
+struct AddNormArgs {
+  bf16_t* residual;        // [M, N], row stride ldr; updated in place
+  const float* norm_w;     // [N]
+  float* partials;         // [M, gridDim.x]
+  long ldr;
+};
+
 // ROWS: weight rows a workgroup owns: 16 fill the MFMA tile; 8 (half the tile idle) give twice
 // the workgroups when N is so small that 16-row tiles would leave CUs without work.
-template <int MT, int U, int ROWS, typename TY>
+// ADD_NORM: the epilogue described at AddNormArgs (MT = 1, bfloat16 output).
+template <int MT, int U, int ROWS, typename TY, bool ADD_NORM = false>
 __global__ void __launch_bounds__(1024)
 gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                   int M, int N, int K, long ldx, long ldy, int k_per_wave) {
+                   int M, int N, int K, long ldx, long ldy, int k_per_wave, AddNormArgs an) {
   extern __shared__ float red[];                 // [waves][MT][64][4]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, lg = lane >> 4;
   const int nwaves = blockDim.x >> 6;
@@ -169,6 +183,25 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
         acc[t] += o;
       }
   }
+  if (ADD_NORM) {
+    const int m = ln;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * lg + i;
+      if (m < M && 4 * lg + i < ROWS && n < N) {
+        // as the separate kernels do it: the product rounded to bfloat16, the sum in float32
+        const float f = round_to<bf16_t>(acc[0][i]) + bf16_to_float(an.residual[(size_t)m * an.ldr + n]);
+        an.residual[(size_t)m * an.ldr + n] = float_to_bf16(f);
+        y[(size_t)m * ldy + n] = from_float<TY>(f * an.norm_w[n]);
+        ss += f * f;
+      }
+    }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if (lg == 0 && m < M) an.partials[(size_t)m * gridDim.x + blockIdx.x] = ss;
+    return;
+  }
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = 16 * t + ln;
@@ -183,7 +216,8 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
 
 template <int MT, int U, int ROWS>
 static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
-                              long ldy, int out_dtype, hipStream_t stream) {
+                              long ldy, int out_dtype, hipStream_t stream,
+                              const AddNormArgs* an = nullptr) {
   const int blocks = (N + ROWS - 1) / ROWS;
   // enough waves to keep every SIMD of 256 CUs busy a few times over, each with
   // at least 256 elements of K to stream
@@ -194,23 +228,32 @@ static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int 
   if (waves < 4 && K >= 1024) waves = 4;
   int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * MT * 64 * 4 * sizeof(float) : 0;
-  if (out_dtype == PTL_DTYPE_F32)
+  if (an != nullptr) {
+    if (MT != 1 || out_dtype != PTL_DTYPE_BF16) return PTL_ERR_ARG;
+    gemm_skinny_kernel<1, U, ROWS, bf16_t, true><<<blocks, waves * 64, lds, stream>>>(
+        (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, *an);
+  } else if (out_dtype == PTL_DTYPE_F32) {
     gemm_skinny_kernel<MT, U, ROWS, float><<<blocks, waves * 64, lds, stream>>>(
-        (float*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave);
-  else
+        (float*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, AddNormArgs{});
+  } else {
     gemm_skinny_kernel<MT, U, ROWS, bf16_t><<<blocks, waves * 64, lds, stream>>>(
-        (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave);
+        (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, AddNormArgs{});
+  }
   return ptl_launch_status();
 }
 
+// weight rows a workgroup of the skinny kernel owns
+static int skinny_rows(int N) { return (N + 15) / 16 <= 160 ? 8 : 16; }
+
 template <int MT, int U>
 static int launch_skinny(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
-                         long ldy, int out_dtype, hipStream_t stream) {
+                         long ldy, int out_dtype, hipStream_t stream,
+                         const AddNormArgs* an = nullptr) {
   // measured on MI355X at K = 2048 and 8192: N = 2048 (128 tiles of 16 rows) gains 10 to 20 %
   // from 8-row tiles, N = 3072 (192 tiles) loses
-  if ((N + 15) / 16 <= 160)
-    return launch_skinny_rows<MT, U, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
-  return launch_skinny_rows<MT, U, 16>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
+  if (skinny_rows(N) == 8)
+    return launch_skinny_rows<MT, U, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, an);
+  return launch_skinny_rows<MT, U, 16>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, an);
 }
 
 extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int M, int N, int K,
@@ -222,6 +265,27 @@ extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int M
   if (M <= 16) return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
   if (M <= 32) return launch_skinny<2, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
   return launch_skinny<4, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
+}
+
+// How many partial sums a row gets from ptl_gemm_skinny_add_norm_bf16 with N columns.
+extern "C" int ptl_gemm_skinny_partials(int N) {
+  const int rows = skinny_rows(N);
+  return (N + rows - 1) / rows;
+}
+
+// y = bf16((x W^T + residual) * norm_w), residual <- x W^T + residual, partials[m][j] = sums of
+// squares of the new residual over column blocks (ptl_gemm_skinny_partials(N) of them a row):
+// see AddNormArgs. M <= 16.
+extern "C" int ptl_gemm_skinny_add_norm_bf16(void* y, const void* x, const void* w, void* residual,
+                                             const float* norm_w, float* partials, int M, int N,
+                                             int K, long ldx, long ldy, long ldr,
+                                             hipStream_t stream) {
+  if (M <= 0 || N <= 0) return PTL_OK;
+  if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldx < K || ldy < N || ldr < N || !residual ||
+      !norm_w || !partials)
+    return PTL_ERR_ARG;
+  const AddNormArgs an = {(bf16_t*)residual, norm_w, partials, ldr};
+  return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, PTL_DTYPE_BF16, stream, &an);
 }
 
 // ===========================================================================
@@ -253,14 +317,32 @@ struct RopeStoreArgs {
   int Hq, Hkv, D, page_size;
 };
 
+// Rows of x that still lack their normalisation factor (see AddNormArgs): the results of row m
+// are multiplied by rsqrt(sum_j partials[m][j] * inv_n + eps). partials == null: no factor.
+struct RowScaleArgs {
+  const float* partials;   // [M, count]
+  int count;
+  float inv_n, eps;
+};
+
 template <int MODE, int U, int ROWS>
 __global__ void __launch_bounds__(1024)
 gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                  int M, int N_out, int K, long ldx, long ldy, int k_per_wave, int pair_offset,
-                 int tiles_per_group, int group_rows, RopeStoreArgs rs) {
+                 int tiles_per_group, int group_rows, RopeStoreArgs rs, RowScaleArgs sc) {
   extern __shared__ float red[];                 // [waves][2][64][4]
+  __shared__ float row_factor[16];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, lg = lane >> 4;
   const int nwaves = blockDim.x >> 6;
+  if (sc.partials != nullptr) {
+    // the waves share the rows; a row's partial sums are added in a fixed order
+    for (int m = wave; m < M; m += nwaves) {
+      float sum = 0.f;
+      for (int j = lane; j < sc.count; j += 64) sum += sc.partials[(size_t)m * sc.count + j];
+      sum = wave_sum(sum);
+      if (lane == 0) row_factor[m] = 1.0f / sqrtf(sum * sc.inv_n + sc.eps);
+    }
+  }
   // workgroup b takes tile (b % tiles_per_group) of group (b / tiles_per_group): rows
   // r1 .. r1+15 and r1 + pair_offset .. of W. SiLU: one group, tiles over I. Rope: a
   // group is a head (group_rows = D), its tiles cover the first half of the head.
@@ -304,6 +386,12 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     }
   }
   const int m = ln;                 // the result tiles hold rows 4*lg+i of W, column m of x^T
+  if (sc.partials != nullptr) {
+    if (nwaves == 1) __syncthreads();            // (more waves: the barrier above was passed)
+    const float f = row_factor[min(m, M - 1)];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { acc1[i] *= f; acc2[i] *= f; }
+  }
   if (m >= M) return;
   if (MODE == PAIR_SILU) {
 #pragma unroll
@@ -354,17 +442,23 @@ static int pair_waves(int blocks, int K) {
 }
 
 // out [M, I] = silu(x Wg^T) * (x Wu^T) for W = [Wg; Wu] of shape [2I, K]; M <= 16, I % 16 == 0
+// partials / n_partials / eps: the normalisation factor of x's rows that is still to be applied
+// (RowScaleArgs; K is the size of the normalised rows); partials == null: none.
 extern "C" int ptl_gate_up_silu_bf16(void* out, const void* x, const void* w, int M, int I, int K,
-                                     long ldx, hipStream_t stream) {
+                                     long ldx, const float* partials, int n_partials, float eps,
+                                     hipStream_t stream) {
   if (M <= 0 || I <= 0) return PTL_OK;
-  if (M > 16 || I % 16 || K <= 0 || K % 8 || ldx % 8 || ldx < K) return PTL_ERR_ARG;
+  if (M > 16 || I % 16 || K <= 0 || K % 8 || ldx % 8 || ldx < K || (partials && n_partials <= 0))
+    return PTL_ERR_ARG;
+  const RowScaleArgs sc = {partials, n_partials, 1.0f / (float)K, eps};
   const int blocks = I / 16;
   const int waves = pair_waves(blocks, K);
   const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
   RopeStoreArgs none = {};
   gemm_pair_kernel<PAIR_SILU, 8, 16><<<blocks, waves * 64, lds, stream>>>(
-      (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, I, K, ldx, I, k_per_wave, I, blocks, 0, none);
+      (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, I, K, ldx, I, k_per_wave, I, blocks, 0, none,
+      sc);
   return ptl_launch_status();
 }
 
@@ -373,11 +467,14 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
                                        int K, long ldx, const int32_t* positions,
                                        const float* inv_freq, const int32_t* slots, void* k_cache,
                                        void* v_cache, int Hq, int Hkv, int D, int page_size,
+                                       const float* partials, int n_partials, float eps,
                                        hipStream_t stream) {
   if (M <= 0) return PTL_OK;
   if (M > 16 || Hq <= 0 || Hkv <= 0 || D <= 0 || D % 32 || K <= 0 || K % 8 || ldx % 8 || ldx < K ||
-      ldq < (long)Hq * D || page_size <= 0 || !positions || (slots && (!k_cache || !v_cache)))
+      ldq < (long)Hq * D || page_size <= 0 || !positions || (slots && (!k_cache || !v_cache)) ||
+      (partials && n_partials <= 0))
     return PTL_ERR_ARG;
+  const RowScaleArgs sc = {partials, n_partials, 1.0f / (float)K, eps};
   // few heads: 8-column tiles, so that twice as many workgroups share the weight stream
   const bool small = (Hq + 2 * Hkv) * (D / 32) <= 160;
   const int tiles = small ? D / 16 : D / 32;      // tiles in half a head
@@ -389,10 +486,10 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
   if (small)
     gemm_pair_kernel<PAIR_ROPE, 8, 8><<<blocks, waves * 64, lds, stream>>>(
         (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,
-        tiles, D, rs);
+        tiles, D, rs, sc);
   else
     gemm_pair_kernel<PAIR_ROPE, 8, 16><<<blocks, waves * 64, lds, stream>>>(
         (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,
-        tiles, D, rs);
+        tiles, D, rs, sc);
   return ptl_launch_status();
 }

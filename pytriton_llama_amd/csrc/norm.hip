@@ -108,3 +108,28 @@ extern "C" int ptl_add_rmsnorm(void* y, const void* x, void* residual, const flo
     return PTL_ERR_ARG;
   return ptl_launch_status();
 }
+
+// y[m, :] = v[m, :] * rsqrt(sum_j partials[m][j] / H + eps): finishes a normalisation whose
+// weight is already in v and whose sums of squares lie in ``count`` partial sums a row (written
+// by the product that made v, see gemm.hip). For consumers that cannot apply the factor to
+// their own results. bfloat16.
+__global__ void __launch_bounds__(256)
+row_scale_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ v,
+                 const float* __restrict__ partials, int count, int H, float eps) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  float sum = 0.f;
+  for (int j = threadIdx.x; j < count; j += blockDim.x) sum += partials[(size_t)m * count + j];
+  sum = block_sum(sum, scratch);
+  const float f = 1.0f / sqrtf(sum / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    y[(size_t)m * H + i] = float_to_bf16(bf16_to_float(v[(size_t)m * H + i]) * f);
+}
+
+extern "C" int ptl_row_scale_bf16(void* y, const void* v, const float* partials, int count, int T_,
+                                  int H, float eps, hipStream_t stream) {
+  if (T_ <= 0) return PTL_OK;
+  if (H <= 0 || count <= 0 || !partials) return PTL_ERR_ARG;
+  row_scale_kernel<<<T_, 256, 0, stream>>>((bf16_t*)y, (const bf16_t*)v, partials, count, H, eps);
+  return ptl_launch_status();
+}

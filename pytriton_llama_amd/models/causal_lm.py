@@ -8,7 +8,7 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from ..parts.base import ParamSource, Part
+from ..parts.base import ParamSource, Part, as_tensor, run_norm
 
 
 @dataclass(frozen=True)
@@ -77,14 +77,24 @@ class CausalLM:
         """Float32 logits [len(ctx.logit_rows), vocab] for the flat batch ``ctx``."""
         h = self.embedding.forward(ctx.token_ids)
         residual = None
-        for call in self.schedule:
+        last = len(self.schedule) - 1
+        for i, call in enumerate(self.schedule):
             cache = storage.view(call.cache_layer, call.writes)
-            h, residual = self.blocks[call.block].forward(h, residual, ctx, cache)
+            block = self.blocks[call.block]
+            # a block may leave its last product to the norm that comes next, if that norm can
+            # take it (parts/base.py); the rows for the final norm are picked first, so not there
+            after = self.blocks[self.schedule[i + 1].block] if i < last else None
+            if (after is not None and getattr(block, "can_defer_output", False)
+                    and getattr(getattr(after, "input_norm", None), "takes_pending_product", False)):
+                h, residual = block.forward(h, residual, ctx, cache, defer_output=True)
+            else:
+                h, residual = block.forward(h, residual, ctx, cache)
+        h = as_tensor(h)
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=h.device)
         if ctx.num_logit_rows != h.shape[0] or not ctx.logit_rows_are_identity:
             h = h.index_select(0, ctx.logit_rows)
             if residual is not None:
                 residual = residual.index_select(0, ctx.logit_rows)
-        h, _ = self.final_norm.forward(h, residual)
-        return self.head.forward(h)
+        h, _ = run_norm(self.final_norm, h, residual)
+        return self.head.forward(as_tensor(h))

@@ -213,6 +213,73 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
 FUSED_MAX_ROWS = 16
 
 
+class RowScale:
+    """The normalisation factor that rows of a tensor still lack: row m is to be multiplied by
+    rsqrt(sum(partials[m]) / size + eps). ``partials`` [M, count] float32 are the sums of squares
+    of the un-normalised row over column blocks (written by ``gemm_skinny_add_norm``)."""
+    __slots__ = ("partials", "size", "eps")
+
+    def __init__(self, partials: torch.Tensor, size: int, eps: float):
+        self.partials, self.size, self.eps = partials, int(size), float(eps)
+
+    def args(self, M: int, K: int, what: str):
+        p = self.partials
+        if (p.dtype != torch.float32 or p.dim() != 2 or p.shape[0] != M or not p.is_contiguous()
+                or not p.is_cuda):
+            raise KernelError(f"{what}: partial sums must be contiguous float32 [{M}, count] on the GPU")
+        if self.size != K:
+            raise KernelError(f"{what}: rows of {K} elements, but the partial sums are of rows of "
+                              f"{self.size}")
+        return _ptr(p), int(p.shape[1]), ctypes.c_float(self.eps)
+
+
+_NO_SCALE = (ctypes.c_void_p(0), 0, ctypes.c_float(0.0))
+
+
+def gemm_skinny_add_norm_fits(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
+                              norm_weight: torch.Tensor) -> bool:
+    return (_fused_x_ok(x, w) and residual.dtype == torch.bfloat16 and residual.is_cuda
+            and residual.dim() == 2 and residual.shape == (x.shape[0], w.shape[0])
+            and residual.stride(1) == 1 and norm_weight.dtype == torch.float32
+            and norm_weight.is_cuda and norm_weight.is_contiguous()
+            and norm_weight.numel() == w.shape[0])
+
+
+def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
+                         norm_weight: torch.Tensor, eps: float):
+    """The product x @ w.T, the residual sum and the part of an RMSNorm that does not need the
+    whole row, in one kernel for at most 16 rows of bfloat16 x (see AddNormArgs in
+    csrc/gemm.hip): ``residual`` becomes x @ w.T + residual in place; returned are
+    y = bfloat16(residual * norm_weight) and the RowScale that y still lacks."""
+    if not gemm_skinny_add_norm_fits(x, w, residual, norm_weight):
+        raise KernelError("gemm_skinny_add_norm: needs bfloat16 x, w, residual [M, N] with M <= 16, "
+                          "K a multiple of 8, aligned rows, a float32 norm weight [N]")
+    M, K = x.shape
+    N = w.shape[0]
+    lib = library.load("gemm")
+    count = int(lib.ptl_gemm_skinny_partials(N))
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    partials = torch.empty((M, count), dtype=torch.float32, device=x.device)
+    _check(lib.ptl_gemm_skinny_add_norm_bf16(
+        _ptr(y), _ptr(x), _ptr(w), _ptr(residual), _ptr(norm_weight), _ptr(partials), M, N, K,
+        ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)), ctypes.c_long(N),
+        ctypes.c_long(residual.stride(0) if M > 1 else N), _stream()), "gemm_skinny_add_norm")
+    return y, RowScale(partials, N, eps)
+
+
+def row_scale(v: torch.Tensor, scale: RowScale) -> torch.Tensor:
+    """v with the factor of ``scale`` applied to its rows (bfloat16 [M, H])."""
+    _need_gpu(v)
+    if v.dtype != torch.bfloat16 or v.dim() != 2 or not v.is_contiguous():
+        raise KernelError("row_scale: needs a contiguous bfloat16 [M, H] tensor")
+    M, H = v.shape
+    pp, count, eps = scale.args(M, H, "row_scale")
+    y = torch.empty_like(v)
+    lib = library.load("norm")
+    _check(lib.ptl_row_scale_bf16(_ptr(y), _ptr(v), pp, count, M, H, eps, _stream()), "row_scale")
+    return y
+
+
 def _fused_x_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return (x.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
             and 0 < x.shape[0] <= FUSED_MAX_ROWS and x.shape[1] % 8 == 0 and x.stride(1) == 1
@@ -224,9 +291,10 @@ def gate_up_silu_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
     return _fused_x_ok(x, w) and w.shape[0] % 32 == 0
 
 
-def gate_up_silu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = None) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) for w = [Wg; Wu] ([2I, K]) and at most 16 rows of
-    bfloat16 x, in one kernel (see csrc/gemm.hip)."""
+    bfloat16 x, in one kernel (see csrc/gemm.hip). ``scale``: the factor that the rows
+    of x still lack; it is applied to both products."""
     if not gate_up_silu_fits(x, w):
         raise KernelError("gate_up_silu: needs bfloat16, at most 16 rows, K a multiple of 8, "
                           "I a multiple of 16, aligned rows")
@@ -234,8 +302,10 @@ def gate_up_silu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     I = w.shape[0] // 2
     out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
     lib = library.load("gemm")
+    pp, count, eps = scale.args(M, K, "gate_up_silu") if scale is not None else _NO_SCALE
     _check(lib.ptl_gate_up_silu_bf16(_ptr(out), _ptr(x), _ptr(w), M, I, K,
-                                     ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)), _stream()),
+                                     ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)),
+                                     pp, count, eps, _stream()),
            "gate_up_silu")
     return out
 
@@ -247,10 +317,12 @@ def qkv_rope_store_fits(x: torch.Tensor, w: torch.Tensor, head_dim: int) -> bool
 def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
                    inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                   num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
+                   num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
+                   scale: Optional[RowScale] = None) -> torch.Tensor:
     """q, k, v = x @ w.T (rows of w: q | k | v), q and k rotated, k and v written
     into the cache pages at ``slots``; returns the rotated q [M, Hq, D]. At most 16
-    rows of bfloat16 x, head sizes in steps of 32 (see csrc/gemm.hip)."""
+    rows of bfloat16 x, head sizes in steps of 32 (see csrc/gemm.hip). ``scale``: the
+    factor that the rows of x still lack; it is applied to the products."""
     if not qkv_rope_store_fits(x, w, head_dim):
         raise KernelError("qkv_rope_store: needs bfloat16, at most 16 rows, K a multiple of 8, "
                           "a head size in steps of 32, aligned rows")
@@ -276,10 +348,12 @@ def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
                                   f"[pages, {Hkv}, {page_size}, {D}]")
     q = torch.empty((M, Hq, D), dtype=torch.bfloat16, device=x.device)
     lib = library.load("gemm")
+    pp, count, eps = scale.args(M, K, "qkv_rope_store") if scale is not None else _NO_SCALE
     _check(lib.ptl_qkv_rope_store_bf16(
         _ptr(q), ctypes.c_long(Hq * D), _ptr(x), _ptr(w), M, K,
         ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)), _ptr(positions), _ptr(inv_freq),
-        _ptr(slots), _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D, int(page_size), _stream()),
+        _ptr(slots), _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D, int(page_size), pp, count, eps,
+        _stream()),
         "qkv_rope_store")
     return q
 

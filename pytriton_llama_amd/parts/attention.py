@@ -7,7 +7,8 @@ from typing import List, Optional
 import torch
 
 from .. import ops
-from .base import PagedKVSpec, ParamSource, Part, place, register_part
+from .base import (PagedKVSpec, ParamSource, Part, PendingProduct, PendingScale, as_tensor, place,
+                   register_part)
 from .linear import LINEAR_LIBRARIES, linear
 
 
@@ -69,18 +70,28 @@ class PagedAttention(Part):
         if self.position is not None:
             self.position.load({}, dtype, device)
 
-    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+    takes_pending_scale = True
+    can_defer_output = True
+
+    def forward(self, x, ctx, cache, defer_output: bool = False):
         T = x.shape[0]
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         group = ctx.groups[cache.group]
         rotary = self.position.rotary_inv_freq() if self.position is not None else None
-        if (self.position is None or rotary is not None) and ops.qkv_rope_store_fits(x, self.qkv, D):
+        fused = self.position is None or rotary is not None
+        scale = None
+        if isinstance(x, PendingScale) and fused and ops.qkv_rope_store_fits(x.values, self.qkv, D):
+            x, scale = x.values, x.scale
+        x = as_tensor(x)
+        if fused and ops.qkv_rope_store_fits(x, self.qkv, D):
             # the few rows of a decode step: projection, rotation and cache write in one kernel
             q = ops.qkv_rope_store(x, self.qkv, ctx.positions, rotary,
                                    group.slots if cache.writable else None, cache.k, cache.v,
-                                   Hq, Hkv, D, cache.page_size)
+                                   Hq, Hkv, D, cache.page_size, scale)
             out = torch.empty((T, Hq, D), dtype=x.dtype, device=x.device)
             self.attend(out, q, cache, ctx, group)
+            if defer_output:
+                return PendingProduct(out.view(T, Hq * D), self.o)
             return linear(out.view(T, Hq * D), self.o)
         qkv = linear(x, self.qkv)
         q = qkv[:, :self.q_size].view(T, Hq, D)

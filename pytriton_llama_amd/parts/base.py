@@ -23,6 +23,23 @@ embedding:       forward(token_ids int32 [T]) -> [T, hidden]
 head:            forward(x [R, hidden]) -> float32 logits [R, vocab]
 block:           forward(h, residual, ctx, cache) -> (h, residual)
 
+Work handed on instead of done (optional; a part that knows nothing of it is given tensors)
+------------------------------------------------------------------------------------------
+For the few rows of a decode step a kernel costs more in starting than in running, so two
+parts may pass each other a value that is not finished yet when the receiver can finish it
+inside a kernel it launches anyway:
+    PendingProduct(x, w)      x @ w.T not computed yet. A mixer or feed-forward whose class
+                              says ``can_defer_output`` returns it for its last projection when
+                              called with defer_output=True; a norm whose class says
+                              ``takes_pending_product`` computes the product, the residual sum
+                              and its own share in one kernel.
+    PendingScale(values, scale)   rows that still lack a factor (the rsqrt of an RMSNorm). A
+                              norm returns it when called with scale_ok=True; a mixer or
+                              feed-forward whose class says ``takes_pending_scale`` applies the
+                              factor to the results of its first product.
+Both have .tensor(), which finishes the work with separate kernels. The block (and the model,
+between blocks) asks the classes for these flags and passes plain tensors to everyone else.
+
 ``ctx`` is the StepContext of engine/batch.py: the flat batch (positions,
 q_start, ctx_len, per cache group its block table and slot mapping, the state
 slot of every sequence). ``cache`` is the view of the one cache layer the call
@@ -61,8 +78,56 @@ class StateSpec:
     dtype: Optional[torch.dtype] = None     # None: the engine dtype
 
 
+class PendingProduct:
+    """x @ w.T that has not been computed (see the module text)."""
+    __slots__ = ("x", "w")
+
+    def __init__(self, x: torch.Tensor, w: torch.Tensor):
+        self.x, self.w = x, w
+
+    @property
+    def shape(self):
+        return (self.x.shape[0], self.w.shape[0])
+
+    def tensor(self) -> torch.Tensor:
+        from .linear import linear
+        return linear(self.x, self.w)
+
+
+class PendingScale:
+    """Rows that still lack a factor (see the module text); ``scale`` is an ops.RowScale."""
+    __slots__ = ("values", "scale")
+
+    def __init__(self, values: torch.Tensor, scale):
+        self.values, self.scale = values, scale
+
+    @property
+    def shape(self):
+        return self.values.shape
+
+    def tensor(self) -> torch.Tensor:
+        from .. import ops
+        return ops.row_scale(self.values, self.scale)
+
+
+def as_tensor(v):
+    """``v`` finished, if it is one of the pending values."""
+    return v.tensor() if isinstance(v, (PendingProduct, PendingScale)) else v
+
+
+def run_norm(norm, x, residual, consumer=None):
+    """norm.forward for an x that may be pending, on behalf of ``consumer`` (the part that gets
+    the result; None: someone who wants a tensor)."""
+    if getattr(norm, "takes_pending_product", False):
+        return norm.forward(x, residual, scale_ok=getattr(consumer, "takes_pending_scale", False))
+    return norm.forward(as_tensor(x), residual)
+
+
 class Part:
     kernel_libraries: Tuple[str, ...] = ()
+    takes_pending_product = False     # norms
+    takes_pending_scale = False       # mixers, feed-forwards
+    can_defer_output = False          # mixers, feed-forwards, blocks
 
     def param_sources(self) -> List[ParamSource]:
         return []

@@ -1,7 +1,7 @@
 """Arrangements of norm, mixer and feed-forward in a block."""
 from __future__ import annotations
 
-from .base import Part, register_part
+from .base import Part, as_tensor, register_part, run_norm
 
 
 @register_part("block", "prenorm")
@@ -27,9 +27,25 @@ class PreNormBlock(Part):
     def cache_spec(self):
         return self.mixer.cache_spec() if hasattr(self.mixer, "cache_spec") else None
 
-    def forward(self, h, residual, ctx, cache):
-        h, residual = self.input_norm.forward(h, residual)
-        h = self.mixer.forward(h, ctx, cache)
-        h, residual = self.post_norm.forward(h, residual)
-        h = self.feed_forward.forward(h)
+    can_defer_output = True
+
+    def forward(self, h, residual, ctx, cache, defer_output: bool = False):
+        """``h`` may be pending work of the block before (parts/base.py); with ``defer_output``
+        the feed-forward may leave its last product to whoever normalises next."""
+        mixer, ffn = self.mixer, self.feed_forward
+        h, residual = run_norm(self.input_norm, h, residual, mixer)
+        if not getattr(mixer, "takes_pending_scale", False):
+            h = as_tensor(h)
+        if (getattr(mixer, "can_defer_output", False)
+                and getattr(self.post_norm, "takes_pending_product", False)):
+            h = mixer.forward(h, ctx, cache, defer_output=True)
+        else:
+            h = mixer.forward(h, ctx, cache)
+        h, residual = run_norm(self.post_norm, h, residual, ffn)
+        if not getattr(ffn, "takes_pending_scale", False):
+            h = as_tensor(h)
+        if defer_output and getattr(ffn, "can_defer_output", False):
+            h = ffn.forward(h, defer_output=True)
+        else:
+            h = ffn.forward(h)
         return h, residual

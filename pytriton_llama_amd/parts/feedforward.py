@@ -6,7 +6,7 @@ from typing import List, Optional
 import torch
 
 from .. import ops
-from .base import ParamSource, Part, place, register_part
+from .base import ParamSource, Part, PendingProduct, PendingScale, as_tensor, place, register_part
 from .linear import LINEAR_LIBRARIES, linear
 
 
@@ -16,7 +16,9 @@ class SwiGLU(Part):
     (lite_llama/models/llama.py:107-120, lite_llama/kernels/swiglu.py:44-67).
     gate and up are concatenated at load into one [2I, hidden] matrix (rows
     gate | up) so that one product feeds the SiLU-multiply kernel."""
-    kernel_libraries = ("activation",) + LINEAR_LIBRARIES
+    kernel_libraries = ("activation", "norm") + LINEAR_LIBRARIES
+    takes_pending_scale = True
+    can_defer_output = True
 
     def __init__(self, hidden_size: int, intermediate_size: int,
                  gate_name: str = "gate_proj.weight", up_name: str = "up_proj.weight",
@@ -37,8 +39,15 @@ class SwiGLU(Part):
         self.gate_up = place(torch.cat([tensors[g], tensors[u]], dim=0), "matrix", dtype, device)
         self.down = place(tensors[d], "matrix", dtype, device)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x, defer_output: bool = False):
+        scale = None
+        if isinstance(x, PendingScale) and ops.gate_up_silu_fits(x.values, self.gate_up):
+            x, scale = x.values, x.scale
+        x = as_tensor(x)
         if ops.gate_up_silu_fits(x, self.gate_up):
             # the few rows of a decode step: product and SiLU-multiply in one kernel
-            return linear(ops.gate_up_silu(x, self.gate_up), self.down)
+            a = ops.gate_up_silu(x, self.gate_up, scale)
+            if defer_output:
+                return PendingProduct(a, self.down)
+            return linear(a, self.down)
         return linear(ops.silu_mul(linear(x, self.gate_up)), self.down)

@@ -6,7 +6,7 @@ from typing import List, Optional
 import torch
 
 from .. import ops
-from .base import ParamSource, Part, place, register_part
+from .base import ParamSource, Part, PendingProduct, PendingScale, as_tensor, place, register_part
 
 
 @register_part("norm", "rmsnorm")
@@ -15,7 +15,8 @@ class RMSNorm(Part):
     sum returned as the new residual (lite_llama/kernels/skip_rmsnorm.py:94-181;
     call sites lite_llama/models/llama.py:149,160,219). Without a residual the
     input itself is the residual (:181)."""
-    kernel_libraries = ("norm",)
+    kernel_libraries = ("norm", "gemm")
+    takes_pending_product = True
 
     def __init__(self, size: int, eps: float, weight_name: str = "weight"):
         self.size = int(size)
@@ -29,6 +30,14 @@ class RMSNorm(Part):
     def load(self, tensors, dtype, device) -> None:
         self.weight = place(tensors[self.weight_name], "vector", dtype, device)
 
-    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor]):
+    def forward(self, x, residual: Optional[torch.Tensor], scale_ok: bool = False):
+        if isinstance(x, PendingProduct):
+            # the few rows of a decode step: the product, the residual sum and the weight in one
+            # kernel; the rsqrt factor is left to the part that takes the result
+            if (scale_ok and residual is not None
+                    and ops.gemm_skinny_add_norm_fits(x.x, x.w, residual, self.weight)):
+                y, scale = ops.gemm_skinny_add_norm(x.x, x.w, residual, self.weight, self.eps)
+                return PendingScale(y, scale), residual
+        x = as_tensor(x)
         y = ops.add_rmsnorm(x, residual, self.weight, self.eps)
         return y, (x if residual is None else residual)

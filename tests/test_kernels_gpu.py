@@ -157,6 +157,79 @@ def test_qkv_rope_store(ops, dims):
     torch.testing.assert_close(q3.float().cpu(), full[:, :Hq * D].view(M, Hq, D), atol=3e-2, rtol=3e-2)
 
 
+@pytest.mark.parametrize("mnk", [(1, 64, 176), (8, 2048, 2048), (16, 136, 320), (5, 4096, 72), (3, 2056, 48)])
+def test_gemm_skinny_add_norm_and_row_scale(ops, mnk):
+    """Product + residual sum + norm weight in one kernel, the rsqrt factor left as partial sums:
+    the residual it leaves, and its output once the factor is applied, are those of the product
+    followed by add_rmsnorm, and of the plain formulas."""
+    M, N, K = mnk
+    torch.manual_seed(12)
+    eps = 1e-5
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    res = torch.randn(M, N, device="cuda").to(torch.bfloat16)
+    nw = (1.0 + 0.2 * torch.randn(N, device="cuda")).float()
+    res_fused = res.clone()
+    y, scale = ops.gemm_skinny_add_norm(x, w, res_fused, nw, eps)
+    assert scale.partials.shape[0] == M and scale.size == N
+    got = ops.row_scale(y, scale)
+    # the separate kernels
+    res_sep = res.clone()
+    want = ops.add_rmsnorm(ops.gemm_skinny(x, w), res_sep, nw, eps)
+    assert torch.equal(res_fused, res_sep)                       # same roundings, same sums
+    torch.testing.assert_close(got.float(), want.float(), atol=3e-2, rtol=2e-2)
+    # the sums of squares against the residual itself
+    ss = scale.partials.sum(dim=1)
+    torch.testing.assert_close(ss, (res_fused.float() ** 2).sum(dim=1), rtol=2e-2, atol=1e-3)
+    # the plain formulas
+    h = (x.double() @ w.double().T).float().cpu() + res.float().cpu()
+    plain, _ = plain_llama.add_rms_norm(h, None, nw.cpu(), eps)
+    torch.testing.assert_close(got.float().cpu(), plain, atol=5e-2, rtol=3e-2)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny_add_norm(torch.zeros(17, K, device="cuda", dtype=torch.bfloat16), w,
+                                 torch.zeros(17, N, device="cuda", dtype=torch.bfloat16), nw, eps)
+    with pytest.raises(ops.KernelError):
+        ops.row_scale(y, ops.RowScale(scale.partials, N + 8, eps))
+
+
+def test_fused_products_apply_a_row_scale(ops):
+    """gate_up_silu and qkv_rope_store with rows that still lack their factor give what they
+    give for the rows with the factor applied."""
+    torch.manual_seed(13)
+    M, H, I, Hq, Hkv, D, P = 6, 328, 176, 4, 2, 32, 8
+    eps = 1e-6
+    v = torch.randn(M, H, device="cuda").to(torch.bfloat16)
+    partials = torch.rand(M, 41, device="cuda") * 30                 # any positive sums do
+    scale = ops.RowScale(partials, H, eps)
+    f = torch.rsqrt(partials.sum(dim=1) / H + eps)
+    xs = (v.float() * f[:, None])                                     # the finished rows, float32
+    wg = (torch.randn(2 * I, H, device="cuda") / math.sqrt(H)).to(torch.bfloat16)
+    got = ops.gate_up_silu(v, wg, scale)
+    gu = xs.double() @ wg.double().T
+    want = (plain_llama.silu(gu[:, :I]) * gu[:, I:]).float()
+    torch.testing.assert_close(got.float(), want, atol=3e-2, rtol=3e-2)
+    wq = (torch.randn((Hq + 2 * Hkv) * D, H, device="cuda") / math.sqrt(H)).to(torch.bfloat16)
+    positions = torch.tensor([0, 3, 9, 100, 2000, 7], dtype=torch.int32, device="cuda")
+    inv_freq = plain_llama.rope_inv_freq_default(10000.0, D).cuda()
+    slots = torch.arange(M, dtype=torch.int32, device="cuda")
+    kc = torch.zeros(2, Hkv, P, D, device="cuda", dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    q = ops.qkv_rope_store(v, wq, positions, inv_freq, slots, kc, vc, Hq, Hkv, D, P, scale)
+    full = (xs.double() @ wq.double().T).float().cpu()
+    cos, sin = plain_llama.rope_cos_sin(inv_freq.cpu(), positions.cpu())
+    want_q = plain_llama.apply_rope(full[:, :Hq * D].view(M, Hq, D), cos, sin)
+    torch.testing.assert_close(q.float().cpu(), want_q, atol=3e-2, rtol=3e-2)
+    want_k = plain_llama.apply_rope(full[:, Hq * D:(Hq + Hkv) * D].view(M, Hkv, D), cos, sin)
+    got_k = kc.view(2 * 1, Hkv, P, D).permute(0, 2, 1, 3).reshape(2 * P, Hkv, D)[:M]
+    torch.testing.assert_close(got_k.float().cpu(), want_k, atol=3e-2, rtol=3e-2)
+    want_v = full[:, (Hq + Hkv) * D:].view(M, Hkv, D)
+    got_v = vc.permute(0, 2, 1, 3).reshape(2 * P, Hkv, D)[:M]
+    torch.testing.assert_close(got_v.float().cpu(), want_v, atol=3e-2, rtol=3e-2)
+    # the factor really is used: without it the result differs
+    q_plain = ops.qkv_rope_store(v, wq, positions, inv_freq, None, None, None, Hq, Hkv, D, P)
+    assert (q_plain.float() - q.float()).abs().max() > 0.1
+
+
 def _rope_reference(x, positions, inv_freq):
     cos, sin = plain_llama.rope_cos_sin(inv_freq, positions)
     return plain_llama.apply_rope(x, cos, sin)
