@@ -214,7 +214,7 @@ def main():
         assert produced == batch * steps, (produced, batch, steps)
         ctx = [engine.requests[i].num_computed for i in ids]
         for i in ids:
-            engine.scheduler.abort(engine.requests.pop(i))
+            engine.abort(i)
         assert not engine.has_work
         mean_ctx = sum(ctx) / len(ctx) - steps / 2.0
         return batch * steps / dt, dt / steps, mean_ctx

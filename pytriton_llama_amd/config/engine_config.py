@@ -42,6 +42,8 @@ class EngineConfig:
     max_model_len: int = 2048                # reference: max_seq_len
     seed: int = 0
     use_graphs: bool = True                  # replay decode-only steps as HIP graphs
+    async_decode: bool = True                # launch a decode step before the tokens of the one
+                                             # before it have reached the host
 
     def __post_init__(self):
         self.dtype = parse_dtype(self.dtype)

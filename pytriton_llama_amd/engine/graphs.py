@@ -130,8 +130,10 @@ class DecodeGraphs:
             b.logits = self.model.forward(b.ctx, self.storage)
         b.graph = graph
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Logits [wanted, vocab] of a step whose entries all bring one token."""
+    def step(self, entries: Sequence[StepEntry], token_feed=None) -> torch.Tensor:
+        """Logits [wanted, vocab] of a step whose entries all bring one token.
+        ``token_feed``: an int32 device tensor with the entries' tokens, for a step that is
+        launched before the host knows them (the entries then carry placeholders)."""
         m = self.manager
         starts = take_pages(entries, m, self.model.vocab_size)
         n = len(entries)
@@ -160,10 +162,14 @@ class DecodeGraphs:
                 else:
                     table_np[i, :len(table)] = table
                 owner[i] = (e.request, len(table))
-        if b.graph is None:
+        def refresh():
             b.dev.copy_(b.host, non_blocking=True)
+            if token_feed is not None:
+                b.view("token_ids")[:n].copy_(token_feed[:n], non_blocking=True)
+        if b.graph is None:
+            refresh()
             self._capture(b)
-        b.dev.copy_(b.host, non_blocking=True)
+        refresh()
         b.graph.replay()
         logits = b.logits
         rows = [i for i, e in enumerate(entries) if e.want]

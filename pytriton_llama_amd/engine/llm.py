@@ -33,6 +33,19 @@ def pages_from_memory(model, engine: EngineConfig) -> int:
     return n
 
 
+class _Launched:
+    """A step that is under way: its plan, the requests that get a token from it (in the order
+    of the token tensors), the tokens on the device and the pinned buffers they are copied to,
+    the event after those copies."""
+    __slots__ = ("plan", "samplers", "tokens", "host_tokens", "want_lp", "host_lps", "done",
+                 "replayed")
+
+    def __init__(self, plan, samplers, tokens, host_tokens, want_lp, host_lps, done, replayed):
+        self.plan, self.samplers, self.tokens = plan, samplers, tokens
+        self.host_tokens, self.want_lp, self.host_lps = host_tokens, want_lp, host_lps
+        self.done, self.replayed = done, replayed
+
+
 class Engine:
     """Model folder (or a config dict with ``random_seed``) -> generated tokens.
 
@@ -65,6 +78,13 @@ class Engine:
         self.sampler = Sampler(ec.seed)
         self.requests: Dict[Hashable, Request] = {}
         self._ids = itertools.count()
+        # a step that has been launched and whose tokens have not been fetched yet; pinned
+        # buffers for the fetches, used in turn (two steps are under way at most)
+        self._inflight: Optional[_Launched] = None
+        self._pinned = [(torch.empty(ec.max_num_seqs, dtype=torch.int32).pin_memory(),
+                         torch.empty(ec.max_num_seqs, dtype=torch.float32).pin_memory())
+                        for _ in range(3)]
+        self._turn = 0
 
     # ---- requests ------------------------------------------------------------
     def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
@@ -82,28 +102,76 @@ class Engine:
         return rid
 
     def step(self) -> List[StepOutput]:
-        """One step of the whole engine: plan, run, sample, record."""
-        plan = self.scheduler.schedule()
+        """One step of the whole engine: plan, run, sample, record. While every running
+        request decodes (and ``async_decode`` is on), the step after this one is launched
+        before this one's tokens are fetched: its tokens travel from the sampler to the model
+        on the device, and the host's planning and book-keeping run beside the GPU's work.
+        Each call still returns the tokens of exactly one step, in order."""
+        if self._inflight is None:
+            self._inflight = self._launch(self.scheduler.schedule(), None)
+        cur, nxt = self._inflight, None
+        if self.config.async_decode and cur.replayed:
+            ahead = self.scheduler.plan_ahead(cur.plan)
+            if ahead is not None:
+                nxt = self._launch(ahead, cur)
+        outs = self._collect(cur)
+        self._inflight = nxt
+        return outs
+
+    def _launch(self, plan, before: Optional["_Launched"]) -> "_Launched":
+        """Start the step ``plan`` and the sampling of its tokens; nothing is waited for.
+        ``before``: the step whose tokens this one consumes while they are still on the device
+        (same requests in the same order, one token each)."""
         entries, samplers = [], []
         for e in plan.entries:
-            toks = e.request.token_slice(e.start, e.num_tokens)
+            toks = [0] if before is not None else e.request.token_slice(e.start, e.num_tokens)
             entries.append(StepEntry(e.request.id, toks, [e.num_tokens - 1] if e.samples else []))
             if e.samples:
                 samplers.append(e.request)
-        logits = self.runner.step(entries)
-        tokens = self.sampler.sample(logits, samplers)
-        logprobs = self.sampler.logprobs(logits, samplers, tokens)
-        outs = self.scheduler.update(plan, {r.id: t for r, t in zip(samplers, tokens)})
-        by_id = {r.id: lp for r, lp in zip(samplers, logprobs) if lp is not None}
-        for o in outs:
-            if o.request in by_id:
-                o.logprob = by_id[o.request]
-                self.requests[o.request].output_logprobs.append(o.logprob)
+        replayed = self.runner.replays(entries)
+        logits = self.runner.step(entries, before.tokens if before is not None else None)
+        ahead = 1 if before is not None else 0
+        tokens = self.sampler.sample_device(logits, samplers, ahead)
+        want_lp, lps = self.sampler.logprobs_device(logits, samplers, tokens)
+        host_tokens, host_lps = self._pinned[self._turn % len(self._pinned)]
+        self._turn += 1
+        n = len(samplers)
+        if n:
+            host_tokens[:n].copy_(tokens, non_blocking=True)
+        if want_lp:
+            host_lps[:len(want_lp)].copy_(lps, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return _Launched(plan, samplers, tokens, host_tokens, want_lp, host_lps, done, replayed)
+
+    def _collect(self, step: "_Launched") -> List[StepOutput]:
+        """Wait for the step's tokens and record them."""
+        step.done.synchronize()
+        n = len(step.samplers)
+        tokens = step.host_tokens[:n].tolist()
+        outs = self.scheduler.update(step.plan, {r.id: t for r, t in zip(step.samplers, tokens)})
+        if step.want_lp:
+            lps = step.host_lps[:len(step.want_lp)].tolist()
+            by_id = {step.samplers[i].id: lp for i, lp in zip(step.want_lp, lps)}
+            for o in outs:
+                if o.request in by_id:
+                    o.logprob = by_id[o.request]
+                    self.requests[o.request].output_logprobs.append(o.logprob)
         return outs
 
     @property
     def has_work(self) -> bool:
-        return self.scheduler.has_work
+        return self.scheduler.has_work or self._inflight is not None
+
+    def abort(self, request_id: Hashable) -> None:
+        """Stop a request: what it holds is given back; a step that is under way still
+        finishes, and what it computed for this request is dropped."""
+        req = self.requests.pop(request_id, None)
+        if req is not None:
+            self.scheduler.abort(req)
+        if self._inflight is not None and not self.scheduler.has_work:
+            self._collect(self._inflight)
+            self._inflight = None
 
     # ---- whole generations ----------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]],

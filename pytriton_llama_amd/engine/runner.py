@@ -41,14 +41,22 @@ class ModelRunner:
         self.storage.clear_slot(slot)
 
     @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def replays(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether this step would run as a captured graph (all entries decode one token)."""
+        return self.graphs is not None and self.graphs.fits(entries)
+
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry], token_feed=None) -> torch.Tensor:
         """Float32 logits [wanted, vocab], in the order of the entries and of
-        their ``want`` lists."""
+        their ``want`` lists. ``token_feed``: the entries' tokens as an int32 device tensor,
+        for a step that replays a graph and is launched before the host knows its tokens."""
         for e in entries:
             if not self.manager.is_live(e.request):
                 self.admit(e.request)
         if self.graphs is not None and self.graphs.fits(entries):
-            logits = self.graphs.step(entries)
+            logits = self.graphs.step(entries, token_feed)
+        elif token_feed is not None:
+            raise ValueError("only steps that replay a graph can take their tokens from the device")
         else:
             ctx, _ = build_context(entries, self.manager, self.device, self.model.vocab_size)
             logits = self.model.forward(ctx, self.storage)

@@ -149,6 +149,33 @@ class Scheduler:
             raise RuntimeError("the scheduler can make no progress: no request fits the free pages")
         return plan
 
+    def plan_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
+        """The step after ``plan``, decided before ``plan``'s tokens are known (its step is
+        running and has taken its pages, ``update`` has not been called for it): possible when
+        ``plan`` decodes every running request, nobody waits, none of them reaches a length
+        limit with the token on its way, and each can get the page it may need. Whether a
+        request stops at an end-of-sequence token is not known yet: it is planned, and
+        ``update`` drops what was computed for it. None when the step has to be planned the
+        ordinary way."""
+        if self.waiting or plan.preempted or len(plan.entries) != len(self.running) or not plan.entries:
+            return None
+        nxt = StepPlan()
+        reserve = [0] * len(self.manager.paged)
+        for e in plan.entries:
+            req = e.request
+            if e.num_tokens != 1 or not e.samples or req.status != RUNNING:
+                return None
+            if len(req.output) + 2 > req.params.max_new_tokens:
+                return None                     # the token on its way is its last
+            if self.max_model_len is not None and req.num_tokens + 2 > self.max_model_len:
+                return None
+            if not self.manager.can_append(req.id, 1, reserve):
+                return None
+            for g, k in enumerate(self.manager.pages_needed(req.id, 1)):
+                reserve[g] += k
+            nxt.entries.append(PlannedEntry(req, e.start + 1, 1, True))
+        return nxt
+
     # ---- after the step ------------------------------------------------------------
     def update(self, plan: StepPlan, sampled: Dict[Hashable, int]) -> List[StepOutput]:
         """Record what the step computed; ``sampled`` maps the id of every entry
@@ -156,6 +183,8 @@ class Scheduler:
         outs: List[StepOutput] = []
         for e in plan.entries:
             req = e.request
+            if req.status == FINISHED:
+                continue            # planned ahead of the token that ended it: nothing to record
             req.num_computed += e.num_tokens
             if not e.samples:
                 continue

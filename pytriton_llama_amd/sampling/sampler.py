@@ -28,46 +28,62 @@ class Sampler:
     def __init__(self, seed: int = 0):
         self.seed = int(seed)
 
-    def logprobs(self, logits: torch.Tensor, requests: Sequence[Request], tokens: Sequence[int]):
-        """log_softmax(logits)[token] for the requests that ask for it (None for the others),
-        from the unscaled logits as the reference does
-        (lite_llama/generete_with_probs.py:154-165)."""
+    def logprobs_device(self, logits: torch.Tensor, requests: Sequence[Request],
+                        tokens: torch.Tensor):
+        """(indices of the requests that ask for log-probabilities, float32 device tensor of
+        log_softmax(logits)[token] for them), from the unscaled logits as the reference does
+        (lite_llama/generete_with_probs.py:154-165); (empty, None) when nobody asks."""
         want = [i for i, r in enumerate(requests) if r.params.logprobs]
-        out = [None] * len(requests)
         if not want:
-            return out
-        rows = logits if len(want) == len(requests) else logits.index_select(
-            0, torch.tensor(want, dtype=torch.int32, device=logits.device))
-        toks = torch.tensor([tokens[i] for i in want], dtype=torch.int32, device=logits.device)
-        for i, lp in zip(want, ops.token_logprob(rows, toks).tolist()):
-            out[i] = lp
+            return want, None
+        if len(want) == len(requests):
+            rows, toks = logits, tokens
+        else:
+            idx = torch.tensor(want, dtype=torch.int32, device=logits.device)
+            rows, toks = logits.index_select(0, idx), tokens.index_select(0, idx)
+        return want, ops.token_logprob(rows, toks.contiguous())
+
+    def logprobs(self, logits: torch.Tensor, requests: Sequence[Request], tokens: Sequence[int]):
+        """As ``logprobs_device`` for tokens on the host: a list with None for the requests that
+        do not ask."""
+        out = [None] * len(requests)
+        toks = torch.tensor(list(tokens), dtype=torch.int32, device=logits.device)
+        want, lp = self.logprobs_device(logits, requests, toks)
+        if want:
+            for i, v in zip(want, lp.tolist()):
+                out[i] = v
         return out
 
-    def sample(self, logits: torch.Tensor, requests: Sequence[Request]) -> List[int]:
-        """logits float32 [R, V], row i for requests[i]; returns R token ids."""
+    def sample_device(self, logits: torch.Tensor, requests: Sequence[Request],
+                      ahead: int = 0) -> torch.Tensor:
+        """logits float32 [R, V], row i for requests[i]; R token ids, int32, on the device (no
+        wait for them). ``ahead``: how many tokens of each request are still on their way and
+        not in its output list yet (they count for the index of the random number)."""
         R = len(requests)
         if logits.shape[0] != R:
             raise ValueError(f"{logits.shape[0]} rows of logits for {R} requests")
         if R == 0:
-            return []
+            return torch.empty((0,), dtype=torch.int32, device=logits.device)
         greedy = [i for i, r in enumerate(requests) if r.params.temperature == 0]
-        drawn = [i for i, r in enumerate(requests) if r.params.temperature != 0]
-        out = [0] * R
         if len(greedy) == R:
-            return ops.argmax(logits).tolist()
-        if greedy:
-            idx = torch.tensor(greedy, dtype=torch.int32, device=logits.device)
-            for i, t in zip(greedy, ops.argmax(logits.index_select(0, idx)).tolist()):
-                out[i] = t
-        rows = logits if len(drawn) == R else logits.index_select(
-            0, torch.tensor(drawn, dtype=torch.int32, device=logits.device))
+            return ops.argmax(logits)
+        drawn = [i for i, r in enumerate(requests) if r.params.temperature != 0]
         params = []
         for i in drawn:
             r = requests[i]
             rs = r.params.seed if r.params.seed is not None else r.id
             params.append((r.params.temperature, r.params.top_p,
-                           uniform_for(self.seed, rs, len(r.output))))
+                           uniform_for(self.seed, rs, len(r.output) + ahead)))
         p = torch.tensor(params, dtype=torch.float32).t().contiguous().to(logits.device)
-        for i, t in zip(drawn, ops.sample_top_p(rows, p[0], p[1], p[2]).tolist()):
-            out[i] = t
+        if len(drawn) == R:
+            return ops.sample_top_p(logits, p[0], p[1], p[2])
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+        gi = torch.tensor(greedy, dtype=torch.int64, device=logits.device)
+        di = torch.tensor(drawn, dtype=torch.int64, device=logits.device)
+        out.index_copy_(0, gi, ops.argmax(logits.index_select(0, gi)))
+        out.index_copy_(0, di, ops.sample_top_p(logits.index_select(0, di), p[0], p[1], p[2]))
         return out
+
+    def sample(self, logits: torch.Tensor, requests: Sequence[Request]) -> List[int]:
+        """As ``sample_device``, waited for: a list of R token ids."""
+        return self.sample_device(logits, requests).tolist()

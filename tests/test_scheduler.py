@@ -132,6 +132,110 @@ def test_eos_and_max_model_len_finish_a_request():
         s.add(Request("e", [], SamplingParams()))
 
 
+def _advance(m, plan):
+    for e in plan.entries:
+        if not m.is_live(e.request.id):
+            m.admit(e.request.id)
+        assert m.append(e.request.id, e.num_tokens) == e.start
+
+
+def test_plan_ahead_only_when_every_running_request_decodes_on():
+    """The step after a decode step can be planned before its tokens are known: only when all
+    running requests decode, nobody waits, no length limit is reached by the token on its way
+    and the pages are there; what was planned for a request that then ends is dropped."""
+    m, s = make(num_pages=16, page=4, seqs=4, budget=32, max_len=64)
+    a, b = req("a", 6, new=4), req("b", 3, new=3)
+    s.add(a)
+    s.add(b)
+    p0 = s.schedule()                                   # both prompts whole
+    _advance(m, p0)
+    assert s.plan_ahead(p0) is None                     # a prompt step: planned the ordinary way
+    s.update(p0, {"a": 5, "b": 6})
+    p1 = s.schedule()                                   # both decode
+    _advance(m, p1)
+    p2 = s.plan_ahead(p1)                               # ... and so they will in the step after
+    assert [(e.request.id, e.start, e.num_tokens, e.samples) for e in p2.entries] == \
+        [("a", 7, 1, True), ("b", 4, 1, True)]
+    _advance(m, p2)                                     # launched before p1's tokens are known
+    s.update(p1, {"a": 5, "b": 7})
+    assert s.plan_ahead(p2) is None                     # b's token on its way (its third) is its last
+    outs = s.update(p2, {"a": 8, "b": 9})
+    assert [(o.request, o.finished) for o in outs] == [("a", False), ("b", True)]
+    # a request that ends at an end-of-sequence token after the next step was planned
+    c = req("c", 2, new=8)
+    s.add(c)
+    p3 = s.schedule()                                   # a decodes, c's prompt
+    _advance(m, p3)
+    assert s.plan_ahead(p3) is None
+    s.update(p3, {"a": 1, "c": 2})                      # (a's fourth token: a ends by length)
+    assert a.status == "finished"
+    d = req("d", 3, new=8)
+    s.add(d)
+    p4 = s.schedule()
+    _advance(m, p4)
+    s.update(p4, {"c": 3, "d": 4})
+    p5 = s.schedule()                                   # c and d decode
+    _advance(m, p5)
+    p6 = s.plan_ahead(p5)
+    assert [e.request.id for e in p6.entries] == ["c", "d"]
+    _advance(m, p6)
+    s.update(p5, {"c": 999, "d": 5})                    # c ends here
+    assert c.status == "finished" and not m.is_live("c")
+    assert s.plan_ahead(p6) is None                     # p6 no longer covers the running requests
+    outs = s.update(p6, {"c": 123, "d": 6})             # what p6 computed for c is dropped
+    assert [(o.request, o.token) for o in outs] == [("d", 6)]
+    assert c.output == [2, 3, 999] and d.output == [4, 5, 6]
+    m.check()
+    # somebody waits: no planning ahead
+    p7 = s.schedule()
+    _advance(m, p7)
+    s.add(req("e", 2, new=2))
+    assert s.plan_ahead(p7) is None
+    # no page for the token after next: no planning ahead
+    m2, s2 = make(num_pages=4, page=4, seqs=2, budget=32)
+    r, other = req("r", 7, new=6), req("o", 5, new=2)
+    s2.add(r)
+    s2.add(other)
+    q0 = s2.schedule()                                  # r: two pages, o: two pages: none is left
+    _advance(m2, q0)
+    s2.update(q0, {"r": 1, "o": 1})
+    q1 = s2.schedule()                                  # r at position 7, the last of its second page
+    _advance(m2, q1)
+    assert m2.paged[0].pool.num_free == 0
+    assert s2.plan_ahead(q1) is None                    # position 8 would need a page that is not there
+
+
+def test_planning_ahead_gives_the_same_outputs():
+    """Driving the scheduler one step ahead wherever it allows gives every request the tokens
+    it gets step by step."""
+    def drive(ahead):
+        m, s = make(num_pages=40, page=4, seqs=4, budget=24, chunk=8, max_len=80)
+        reqs = [req(i, n, new=k) for i, (n, k) in enumerate([(5, 9), (17, 4), (9, 12), (3, 7)])]
+        for r in reqs[:3]:
+            s.add(r)
+        pending, steps, late = None, 0, reqs[3]
+        while s.has_work or pending is not None:
+            if pending is None:
+                pending = s.schedule()
+                _advance(m, pending)
+            cur, nxt = pending, None
+            if ahead:
+                nxt = s.plan_ahead(cur)
+                if nxt is not None:
+                    _advance(m, nxt)
+            toks = {e.request.id: (e.start * 7 + 3) % 50 for e in cur.entries if e.samples}
+            s.update(cur, toks)
+            m.check()
+            pending = nxt
+            steps += 1
+            if steps == 6:
+                s.add(late)
+            assert steps < 500
+        assert m.paged[0].pool.num_free == 40
+        return [r.output for r in reqs]
+    assert drive(True) == drive(False)
+
+
 def test_a_request_that_can_never_fit_is_refused():
     m, s = make(num_pages=4, page=4)
     with pytest.raises(ValueError, match="never fit"):
