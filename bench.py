@@ -161,7 +161,8 @@ def main():
                       max_num_seqs=max_batch, max_num_batched_tokens=max(S, 2048),
                       max_model_len=S + W + K + slack, seed=0)
     t0 = time.time()
-    log(f"building the {cfg['num_hidden_layers']}-layer 1B-shape model with random weights ({args.dtype})")
+    log(f"building the {cfg['num_hidden_layers']}-layer {args.shape.upper()}-shape model with random weights "
+        f"({args.dtype})")
     engine = Engine(cfg, ec, random_seed=0)
     log(f"model ready in {time.time() - t0:.1f}s")
     g = torch.Generator().manual_seed(1234)
