@@ -29,8 +29,10 @@
 // V[key0 + 0..3][d0 + l]. Softmax is the online one of
 // lite_llama/kernels/flashattentionv2.py:10-61 in base 2 (scale * log2 e folded
 // into the scores, exp2), float32 max / denominator / accumulator; P is rounded
-// to bfloat16 for the second product as there (:55).
-// Needs D % 32 == 0, D <= 128.
+// to bfloat16 for the second product as there (:55). The running maximum is a
+// stabiliser, not a result: it follows the scores only when they pass it by more
+// than 8 (in the exponent's units), so that what is kept is rescaled rarely.
+// Needs D % 32 == 0, D <= 128, a page size that is a power of two.
 // ===========================================================================
 
 #define PF_BN 64
@@ -103,15 +105,27 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
   const int wave_min_q = first_q + (wave_has_rows ? wave_first_row : 0);
   const int wave_max_q = first_q + min(rows, wave_first_row + 16 * RT) - 1;
 
-  f32x4_t o[RT][2 * NDT];
+  // The softmax denominator. 16 rows a wave (registers to spare): o[r][2 NDT] is one more tile
+  // of the second product, whose "values" are all one; it sums the probabilities as the product
+  // sees them (rounded to bfloat16; float32 sums) and is rescaled with the numerators. 32 rows
+  // a wave: every lane adds its probabilities (float32) and the lanes of a column meet at the end.
+  constexpr bool L_MFMA = RT == 1;
+  f32x4_t o[RT][2 * NDT + 1];
   float m_run[RT], l_part[RT];
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
     m_run[r] = -INFINITY;
     l_part[r] = 0.f;
 #pragma unroll
-    for (int t = 0; t < 2 * NDT; ++t) o[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t <= 2 * NDT; ++t) o[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
+  Frag8 ones;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) ones.v[j] = (__bf16)1.0f;
+  // the running maximum follows the scores only when they pass it by more than this (raw
+  // units): until then exp2 of a score minus the maximum stays below 2^8, which float32 sums
+  // and bfloat16 probabilities hold as well as values below 1, and nothing is rescaled
+  const float lazy = 8.0f / scale_log2;
 
   const int k_end = min(ctx, first_q + rows);
   const int k_lo = window > 0 ? max(0, first_q - window + 1) : 0;
@@ -224,20 +238,20 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
       float tmax = max2(max2(tm[0], tm[1]), max2(tm[2], tm[3]));
       tmax = max2(tmax, lane_xor(tmax, xor16));
       tmax = max2(tmax, lane_xor(tmax, xor32));
-      const float m_new = max2(m_run[r], tmax);
-      const float m_safe = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
-      // the max moved for this lane's row: rescale what is kept. (A branch per lane, not per
-      // wave: the lanes that skip it keep their registers, so nothing is copied where it joins.)
-      if (m_new > m_run[r]) {
-        const float alpha = __builtin_amdgcn_exp2f((m_run[r] - m_safe) * scale_log2);
+      // the maximum moved far enough for this lane's row: rescale what is kept. (A branch per
+      // lane, not per wave: the lanes that skip it keep their registers, so nothing is copied
+      // where it joins.)
+      if (tmax > m_run[r] + lazy) {
+        const float alpha = __builtin_amdgcn_exp2f((m_run[r] - tmax) * scale_log2);
+        m_run[r] = tmax;
         l_part[r] *= alpha;
 #pragma unroll
-        for (int t = 0; t < 2 * NDT; ++t) {
+        for (int t = 0; t < 2 * NDT + (L_MFMA ? 1 : 0); ++t) {
           o[r][t][0] *= alpha; o[r][t][1] *= alpha; o[r][t][2] *= alpha; o[r][t][3] *= alpha;
         }
       }
-      m_run[r] = m_new;
-      const float mc = -m_safe * scale_log2;
+      // (a row that has seen no key yet and sees none in this tile: all its scores are -inf)
+      const float mc = (MASKED && m_run[r] == -INFINITY) ? 0.f : -m_run[r] * scale_log2;
 #pragma unroll
       for (int half = 0; half < 2; ++half)
 #pragma unroll
@@ -245,7 +259,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const float p = __builtin_amdgcn_exp2f(fmaf(st[r][2 * half + t][i], scale_log2, mc));
-            l_part[r] += p;
+            if (!L_MFMA) l_part[r] += p;
             pb[r][half].v[4 * t + i] = (__bf16)p;
           }
     }
@@ -263,6 +277,13 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
         for (int r = 0; r < RT; ++r)
           o[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb[r][half].v, o[r][dt], 0, 0, 0);
       }
+    if (L_MFMA) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+          o[r][2 * NDT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[r][half].v, o[r][2 * NDT], 0, 0, 0);
+    }
   };
 
   load_pages(0);
@@ -292,8 +313,11 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
 
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
-    float l = l_part[r] + __shfl_xor(l_part[r], 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    float l = o[r][2 * NDT][0];                // every row of that tile holds the column's sum
+    if (!L_MFMA) {
+      l = l_part[r] + __shfl_xor(l_part[r], 16, 64);
+      l += __shfl_xor(l, 32, 64);
+    }
     if (row_ok[r]) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;
       const int my_row = 16 * (RT * wave + r) + ln;

@@ -30,6 +30,51 @@ def test_rmsnorm_part(gpu_device):
     assert res0 is xc
 
 
+def test_pending_values_between_parts(gpu_device):
+    """A product left undone goes into the norm's kernel, the norm's rsqrt factor into the next
+    product: a feed-forward -> norm -> feed-forward chain built that way gives what the parts give
+    with finished tensors in between; a receiver that knows nothing of it gets tensors."""
+    from pytriton_llama_amd.parts import build_part
+    from pytriton_llama_amd.parts.base import PendingProduct, PendingScale, as_tensor, run_norm
+    torch.manual_seed(3)
+    H, I, M = 136, 208, 5
+    ff1 = build_part("feed_forward", "swiglu", hidden_size=H, intermediate_size=I)
+    ff2 = build_part("feed_forward", "swiglu", hidden_size=H, intermediate_size=I)
+    for ff in (ff1, ff2):
+        ff.load({"gate_proj.weight": 0.1 * torch.randn(I, H), "up_proj.weight": 0.1 * torch.randn(I, H),
+                 "down_proj.weight": 0.1 * torch.randn(H, I)}, torch.bfloat16, gpu_device)
+    norm = build_part("norm", "rmsnorm", size=H, eps=1e-5)
+    norm.load({"weight": 1 + 0.2 * torch.randn(H)}, torch.bfloat16, gpu_device)
+    x = torch.randn(M, H, device="cuda").to(torch.bfloat16)
+    res = torch.randn(M, H, device="cuda").to(torch.bfloat16)
+    # finished tensors everywhere
+    r_plain = res.clone()
+    y1 = ff1.forward(x)
+    n1, r_plain = norm.forward(y1, r_plain)
+    want = ff2.forward(n1)
+    # work handed on
+    r_lazy = res.clone()
+    p = ff1.forward(x, defer_output=True)
+    assert isinstance(p, PendingProduct) and p.shape == (M, H)
+    torch.testing.assert_close(p.tensor().float(), y1.float(), atol=1e-2, rtol=1e-2)
+    s, r_lazy = run_norm(norm, p, r_lazy, consumer=ff2)
+    assert isinstance(s, PendingScale)
+    assert torch.equal(r_lazy, r_plain)
+    torch.testing.assert_close(s.tensor().float(), n1.float(), atol=3e-2, rtol=2e-2)
+    got = ff2.forward(s)
+    torch.testing.assert_close(got.float(), want.float(), atol=3e-2, rtol=3e-2)
+    # a consumer without the flag, and no consumer: the norm finishes its work itself
+    toy = build_part("feed_forward", "toy_relu", hidden_size=H, inner=64)
+    r3 = res.clone()
+    t, r3 = run_norm(norm, ff1.forward(x, defer_output=True), r3, consumer=toy)
+    assert isinstance(t, torch.Tensor) and torch.equal(r3, r_plain)
+    torch.testing.assert_close(t.float(), n1.float(), atol=3e-2, rtol=2e-2)
+    assert as_tensor(t) is t
+    # float32 and many rows never defer
+    many = torch.randn(40, H, device="cuda").to(torch.bfloat16)
+    assert isinstance(ff1.forward(many, defer_output=True), torch.Tensor)
+
+
 def test_rotary_part_alone(gpu_device):
     from pytriton_llama_amd.parts import build_part
     sc = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
