@@ -125,6 +125,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other batch sizes to report, '' for none")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-probes", action="store_true",
+                    help="skip the two probes of the box (streaming read, MFMA loop)")
     ap.add_argument("--prefill-only", action="store_true", help="measure the prefill and stop (for profiles)")
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES),
                     help="layer sizes: the default 1b is the benchmark; 3b and 8b are the secondary shapes")
@@ -251,8 +253,41 @@ def main():
     }
     if prefill is not None:
         out["prefill"] = prefill
+    if not args.no_probes and args.dtype == "bfloat16":
+        # what this box gives beside the published peaks the fractions above are taken of
+        peaks = measured_peaks()
+        out["measured_peaks"] = peaks
+        out["roofline"]["frac_of_measured"] = round(achieved / peaks["hbm_read_gbs"], 4)
+        log(f"probes: streaming read {peaks['hbm_read_gbs']:.0f} GB/s, bf16 MFMA loop "
+            f"{peaks['mfma_bf16_tflops']:.0f} TFLOP/s")
     print(json.dumps(out), flush=True)
     return 0
+
+
+def measured_peaks():
+    """Streaming-read bandwidth (1 GiB that no cache holds, read by a kernel that does nothing
+    else, one workgroup a CU) and the rate of a loop of independent bfloat16 MFMAs (eight
+    workgroups of four waves a CU)."""
+    import torch
+    from pytriton_llama_amd import ops
+    buf = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").zero_()
+
+    def timed(f, reps):
+        f()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            f()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e-3 / reps
+
+    t = timed(lambda: ops.probe_stream_read(buf, 256), 5)      # one workgroup a CU reads fastest
+    iters, blocks = 4096, 2048
+    t2 = timed(lambda: ops.probe_mfma(iters, blocks), 3)
+    return {"hbm_read_gbs": round(buf.numel() / t / 1e9, 1),
+            "mfma_bf16_tflops": round(blocks * iters * ops.PROBE_MFMA_FLOPS_PER_ITER / t2 / 1e12, 1)}
 
 
 if __name__ == "__main__":

@@ -566,3 +566,25 @@ def token_logprob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
     _check(lib.ptl_token_logprob(_ptr(out), _ptr(logits), _ptr(tokens), R, V,
                                  ctypes.c_long(logits.stride(0)), _stream()), "token_logprob")
     return out
+
+
+def probe_stream_read(buf: torch.Tensor, blocks: int = 512) -> None:
+    """Launch the kernel that only reads ``buf`` (see csrc/probe.hip); time it from outside."""
+    _need_gpu(buf)
+    if not buf.is_contiguous() or buf.data_ptr() % 16:
+        raise KernelError("probe_stream_read: a contiguous, 16-byte aligned tensor")
+    sink = torch.empty(blocks * 256, dtype=torch.int32, device=buf.device)
+    lib = library.load("probe")
+    _check(lib.ptl_probe_stream_read(_ptr(buf), ctypes.c_size_t(buf.numel() * buf.element_size()),
+                                     int(blocks), _ptr(sink), _stream()), "probe_stream_read")
+
+
+PROBE_MFMA_FLOPS_PER_ITER = 4 * 8 * 16 * 16 * 32 * 2      # per workgroup of four waves
+
+
+def probe_mfma(iters: int, blocks: int, device="cuda") -> None:
+    """Launch ``blocks`` workgroups of four waves that each issue ``iters`` * 8 independent
+    bfloat16 MFMAs (see csrc/probe.hip): blocks * iters * PROBE_MFMA_FLOPS_PER_ITER operations."""
+    out = torch.empty(blocks * 256, dtype=torch.float32, device=device)
+    lib = library.load("probe")
+    _check(lib.ptl_probe_mfma(_ptr(out), int(iters), int(blocks), _stream()), "probe_mfma")
