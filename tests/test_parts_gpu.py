@@ -243,3 +243,78 @@ def test_toy_state_mixer_beside_windowed_attention(gpu_device):
            {"r2": seqs["r2"]})
     held = sum(p >= 0 for p in runner.manager.block_table("r2", 0))
     assert held <= 24 // 8 + 2 < len(runner.manager.block_table("r2", 0))
+
+
+ROUTED = {"architectures": ["ToyStateLM"], "vocab_size": 80, "hidden_size": 40, "inner": 24, "experts": 5,
+          "layers": ["attention", "state", "attention"], "order": [0, 1, 2], "decay": 0.8, "heads": 5,
+          "kv_heads": 1, "head_dim": 16, "toy_norm": True, "toy_ffn": True, "toy_position": True,
+          "initializer_range": 0.25}
+
+
+def routed_plain(model, ids):
+    """Whole-sequence logits of the ROUTED toy model, no cache, formulas spelt out here."""
+    ids = torch.as_tensor(ids)
+    S = len(ids)
+    h, residual = model.embedding.weight.float().cpu()[ids], None
+    for call in model.schedule:
+        b = model.blocks[call.block]
+        s = h if residual is None else h + residual
+        h, residual = s - s.mean(-1, keepdim=True), s
+        m = b.mixer
+        if hasattr(m, "decay"):
+            u = h @ m.w.float().cpu().T
+            st = torch.zeros(u.shape[1])
+            ys = []
+            for t in range(S):
+                st = m.decay * st + u[t]
+                ys.append(st)
+            h = torch.stack(ys)
+        else:
+            qkv = h @ m.qkv.float().cpu().T
+            q = qkv[:, :m.q_size].view(S, m.num_heads, m.head_dim)
+            k = qkv[:, m.q_size:m.q_size + m.kv_size].view(S, m.num_kv_heads, m.head_dim)
+            v = qkv[:, m.q_size + m.kv_size:].view(S, m.num_kv_heads, m.head_dim)
+            f = torch.exp(torch.arange(S).float()[:, None, None] * m.position.log_g[None, None, :])
+            o = plain_llama.causal_attention(q * f, k / f, v, m.scale)
+            h = o.reshape(S, -1) @ m.o.float().cpu().T
+        s = h + residual
+        h, residual = s - s.mean(-1, keepdim=True), s
+        ff = b.feed_forward
+        logits = h @ ff.router.cpu().T
+        out = torch.zeros_like(h)
+        for t in range(S):
+            top, idx = logits[t].topk(2)
+            mix = torch.softmax(top, dim=-1)
+            for slot in range(2):
+                e = int(idx[slot])
+                out[t] += mix[slot] * (torch.relu(h[t] @ ff.w1[e].float().cpu().T) @ ff.w2[e].float().cpu().T)
+        h = out
+    s = h + residual
+    h = s - s.mean(-1, keepdim=True)
+    return h @ model.head.weight.float().cpu().T
+
+
+def test_toy_routed_feed_forward_and_toy_position_encoding(gpu_device):
+    """A feed-forward with routing (five experts, two per token) and a position encoding that is
+    no rotation, both defined in the tests, in a model with paged attention and a state mixer:
+    all cuttings agree with the plain whole-sequence result."""
+    from pytriton_llama_amd.config import build_model
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_random_weights
+    model = build_model(copy.deepcopy(ROUTED))
+    load_random_weights(model, 4, torch.float32, gpu_device)
+    g = torch.Generator().manual_seed(8)
+    seqs = {f"r{i}": torch.randint(0, 80, (n,), generator=g).tolist() for i, n in enumerate([66, 40, 97, 51])}
+    want = {rid: routed_plain(model, t) for rid, t in seqs.items()}
+    # every expert is used by some token, or the routing is not tested
+    ff = model.blocks[0].feed_forward
+    x = model.embedding.weight[torch.tensor(seqs["r2"], device="cuda")]
+    assert len(set((x.float() @ ff.router.T).topk(2, dim=-1).indices.flatten().tolist())) == 5
+    for steps in (cuttings.whole(seqs), cuttings.tail_decode(seqs, 32), cuttings.portions(seqs),
+                  cuttings.mixed(seqs, seed=3)):
+        runner = ModelRunner(model, page_size=8, num_pages=48, max_num_seqs=4)
+        got = replay(runner, steps, seqs)
+        for rid in seqs:
+            err = (got[rid] - want[rid]).abs().max() / float(want[rid].abs().max())
+            assert err < 2e-4, (rid, float(err))
+        assert runner.manager.paged[0].pool.num_free == 48

@@ -1,6 +1,7 @@
 """Parts defined by the tests, in plain torch, registered like any other part:
-they show that a mixer with state of its own, another feed-forward, norm,
-position scheme or whole architecture needs no change to the package's files.
+they show that a mixer with state of its own, another feed-forward (also one with
+routing), norm, position encoding or whole architecture needs no change to the
+package's files.
 They are toys, not a model of anyone's."""
 import torch
 
@@ -86,6 +87,64 @@ class ToyRelu(Part):
         return torch.relu(x @ self.w1.T) @ self.w2.T
 
 
+@register_part("feed_forward", "toy_routed")
+class ToyRouted(Part):
+    """A feed-forward with routing: router logits in float32, the two best experts of every
+    token, their outputs mixed by the softmax over the two logits. Experts are small ReLU
+    networks kept in one stacked tensor."""
+
+    def __init__(self, hidden_size, inner, experts):
+        self.hidden_size, self.inner, self.experts = hidden_size, inner, experts
+
+    def param_sources(self):
+        E, H, I = self.experts, self.hidden_size, self.inner
+        return [ParamSource("router", (E, H)), ParamSource("w1", (E * I, H)),
+                ParamSource("w2", (E * H, I))]
+
+    def load(self, tensors, dtype, device):
+        E, H, I = self.experts, self.hidden_size, self.inner
+        self.router = place(tensors["router"], "matrix", dtype, device).float()
+        self.w1 = place(tensors["w1"], "matrix", dtype, device).view(E, I, H)
+        self.w2 = place(tensors["w2"], "matrix", dtype, device).view(E, H, I)
+
+    def forward(self, x):
+        logits = x.float() @ self.router.T                                   # [T, E]
+        top, idx = logits.topk(2, dim=-1)
+        mix = torch.softmax(top, dim=-1)
+        y = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        for e in range(self.experts):
+            for slot in range(2):
+                rows = (idx[:, slot] == e).nonzero().flatten()
+                if rows.numel():
+                    xe = x[rows].float()
+                    ye = torch.relu(xe @ self.w1[e].float().T) @ self.w2[e].float().T
+                    y[rows] += mix[rows, slot, None] * ye
+        return y.to(x.dtype)
+
+
+@register_part("position", "toy_decay")
+class ToyDecayPosition(Part):
+    """Another position encoding, not a rotation: q is multiplied by g_j ** p and k by
+    g_j ** -p (g_j a little below 1, one per element of the head), so a score depends on the
+    distance of the two positions only and far keys fade. It takes the path of position parts
+    that are not rotary: ``rotary_inv_freq`` is None and ``apply`` changes q and k in place."""
+
+    def __init__(self, head_dim, strength):
+        self.head_dim, self.strength = head_dim, strength
+        self.log_g = -strength * torch.arange(1, head_dim + 1, dtype=torch.float32) / head_dim
+
+    def load(self, tensors, dtype, device):
+        self.log_g_dev = self.log_g.to(device)
+
+    def rotary_inv_freq(self):
+        return None
+
+    def apply(self, q, k, positions):
+        f = torch.exp(positions.float()[:, None, None] * self.log_g_dev[None, None, :])
+        q.copy_((q.float() * f).to(q.dtype))
+        k.copy_((k.float() / f).to(k.dtype))
+
+
 @register_part("head", "toy_head")
 class ToyHead(Part):
     def __init__(self, vocab_size, hidden_size):
@@ -121,14 +180,22 @@ def build_toy(cfg: ToyConfig) -> CausalLM:
         if kind == "state":
             mixer = build_part("mixer", "toy_decay_state", hidden_size=H, decay=cfg.decay)
         else:
-            pos = build_part("position", "rotary", head_dim=cfg.head_dim, theta=100.0)
+            if getattr(cfg, "toy_position", False):
+                pos = build_part("position", "toy_decay", head_dim=cfg.head_dim, strength=0.02)
+            else:
+                pos = build_part("position", "rotary", head_dim=cfg.head_dim, theta=100.0)
             mixer = build_part("mixer", "paged_attention", hidden_size=H, num_heads=cfg.heads,
                                num_kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, position=pos,
                                window=getattr(cfg, "window", None))
         norm_name, norm_kw = (("toy_meannorm", dict(size=H)) if cfg.toy_norm
                               else ("rmsnorm", dict(size=H, eps=1e-5)))
-        ffn = (build_part("feed_forward", "toy_relu", hidden_size=H, inner=cfg.inner) if cfg.toy_ffn
-               else build_part("feed_forward", "swiglu", hidden_size=H, intermediate_size=cfg.inner))
+        if getattr(cfg, "experts", 0):
+            ffn = build_part("feed_forward", "toy_routed", hidden_size=H, inner=cfg.inner,
+                             experts=cfg.experts)
+        elif cfg.toy_ffn:
+            ffn = build_part("feed_forward", "toy_relu", hidden_size=H, inner=cfg.inner)
+        else:
+            ffn = build_part("feed_forward", "swiglu", hidden_size=H, intermediate_size=cfg.inner)
         b = build_part("block", "prenorm", input_norm=build_part("norm", norm_name, **norm_kw),
                        mixer=mixer, post_norm=build_part("norm", norm_name, **norm_kw), feed_forward=ffn)
         blocks.append(b)
