@@ -239,3 +239,49 @@ def test_steps_launched_ahead_give_the_same_tokens(folder_b, dtype):
     stop_ahead, _, n2 = run(True, eos)
     assert stop_plain[0] == (plain_out[0][0][:cut], "eos")
     assert stop_ahead == stop_plain and n2 > 5
+
+
+def test_random_traffic_with_and_without_steps_ahead(folder_a):
+    """Forty requests of random lengths arriving at random steps, greedy and sampled, some ending
+    at an end-of-sequence token, with so few pages that requests are preempted: every request
+    gets the same tokens and the same finish reason whether steps are launched ahead or not, and
+    no page or slot is lost."""
+    from pytriton_llama_amd.config import EngineConfig
+    from pytriton_llama_amd.engine import Engine, SamplingParams
+    import random
+    folder, page = folder_a
+
+    def run(async_decode):
+        rng = random.Random(11)
+        g = torch.Generator().manual_seed(12)
+        eng = Engine(folder, EngineConfig(dtype="float32", page_size=page, num_pages=36, max_num_seqs=6,
+                                          max_num_batched_tokens=48, prefill_chunk=16, max_model_len=72,
+                                          seed=5, async_decode=async_decode))
+        eng.scheduler.eos_token_ids = (7, 91, 200)
+        todo, done, ahead = [], {}, 0
+        for i in range(40):
+            n = rng.randint(2, 30)
+            sp = SamplingParams(temperature=rng.choice([0.0, 0.0, 0.8]), top_p=rng.choice([1.0, 0.9]),
+                                max_new_tokens=rng.randint(1, 24), seed=1000 + i)
+            todo.append((rng.randint(0, 60), torch.randint(0, 256, (n,), generator=g).tolist(), sp, i))
+        todo.sort(key=lambda t: t[0])
+        step = 0
+        while todo or eng.has_work:
+            while todo and todo[0][0] <= step:
+                _, prompt, sp, i = todo.pop(0)
+                eng.add_request(prompt, sp, request_id=i)
+            if eng.has_work:
+                eng.step()
+                ahead += eng._inflight is not None
+            step += 1
+            assert step < 5000
+        eng.runner.manager.check()
+        assert eng.runner.manager.paged[0].pool.num_free == 36 and eng.runner.manager.num_free_slots == 6
+        return {i: (r.output, r.finish_reason) for i, r in eng.requests.items()}, ahead, \
+            eng.scheduler.num_preemptions
+
+    plain, n0, p0 = run(False)
+    fast, n1, p1 = run(True)
+    assert len(plain) == 40 and n0 == 0 and n1 > 0
+    assert fast == plain
+    assert {r for _, r in plain.values()} >= {"length", "eos"}
