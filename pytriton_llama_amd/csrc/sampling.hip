@@ -122,6 +122,23 @@ __device__ __forceinline__ float block_exclusive_scan(float v, float* tmp, float
   return tmp[wave] + inc - v;
 }
 
+// Every pass over a row: four consecutive values a thread and step (one 16-byte load) when the
+// row is 16-byte aligned, then the few values that are left; f(i, value).
+template <typename F>
+__device__ __forceinline__ void for_row(const float* __restrict__ p, int V, bool vec, F f) {
+  if (vec) {
+    const int n4 = V >> 2;
+    const float4* p4 = reinterpret_cast<const float4*>(p);
+    for (int i = threadIdx.x; i < n4; i += blockDim.x) {
+      const float4 v = p4[i];
+      f(4 * i, v.x); f(4 * i + 1, v.y); f(4 * i + 2, v.z); f(4 * i + 3, v.w);
+    }
+    for (int i = 4 * n4 + threadIdx.x; i < V; i += blockDim.x) f(i, p[i]);
+  } else {
+    for (int i = threadIdx.x; i < V; i += blockDim.x) f(i, p[i]);
+  }
+}
+
 // work: float [R, V] scratch of the caller; it receives exp(logit/T - max) in the second
 // pass, which the later passes read back instead of computing it again, and in the end (if
 // want_probs) the renormalised nucleus distribution.
@@ -147,15 +164,35 @@ sample_top_p_kernel(int32_t* __restrict__ out, float* __restrict__ work, int wan
   const float inv_t = 1.0f / temperature[r];
   const float c = inv_t * 1.4426950408889634f;
 
+  const bool vec_in = (((uintptr_t)row) & 15) == 0, vec_ex = (((uintptr_t)ex) & 15) == 0;
   float mx = -INFINITY;
-  for (int i = tid; i < V; i += SMP_THREADS) mx = fmaxf(mx, row[i]);
+  for_row(row, V, vec_in, [&](int, float x) { mx = fmaxf(mx, x); });
   mx = block_max(mx, scratch);
   const float mc = mx * c;
   float z = 0.f;
-  for (int i = tid; i < V; i += SMP_THREADS) {
-    const float e = __builtin_amdgcn_exp2f(fmaf(row[i], c, -mc));
-    ex[i] = e;
-    z += e;
+  if (vec_in && vec_ex) {
+    const int n4 = V >> 2;
+    for (int i = tid; i < n4; i += SMP_THREADS) {
+      const float4 x = reinterpret_cast<const float4*>(row)[i];
+      float4 e;
+      e.x = __builtin_amdgcn_exp2f(fmaf(x.x, c, -mc));
+      e.y = __builtin_amdgcn_exp2f(fmaf(x.y, c, -mc));
+      e.z = __builtin_amdgcn_exp2f(fmaf(x.z, c, -mc));
+      e.w = __builtin_amdgcn_exp2f(fmaf(x.w, c, -mc));
+      reinterpret_cast<float4*>(ex)[i] = e;
+      z += (e.x + e.y) + (e.z + e.w);
+    }
+    for (int i = 4 * n4 + tid; i < V; i += SMP_THREADS) {
+      const float e = __builtin_amdgcn_exp2f(fmaf(row[i], c, -mc));
+      ex[i] = e;
+      z += e;
+    }
+  } else {
+    for (int i = tid; i < V; i += SMP_THREADS) {
+      const float e = __builtin_amdgcn_exp2f(fmaf(row[i], c, -mc));
+      ex[i] = e;
+      z += e;
+    }
   }
   z = block_sum(z, scratch);                 // (its barriers also publish ex[] to the block)
   const float tp = top_p[r] * z;             // all masses below are in units of e
@@ -182,15 +219,14 @@ sample_top_p_kernel(int32_t* __restrict__ out, float* __restrict__ work, int wan
       lo[round] = lo_d;
       inv_w[round] = 1.0f / width;
       for (int b = 0; b < SMP_FAN; ++b) cols[b * SMP_THREADS + tid] = 0.f;
-      for (int i = tid; i < V; i += SMP_THREADS) {
-        const float e = ex[i];
+      for_row(ex, V, vec_ex, [&](int, float e) {
         const float d = fmaxf(-__builtin_amdgcn_logf(e) * 0.6931471805599453f, 0.f);   // e may be a hair above 1
         bool in = true;
 #pragma unroll
         for (int q = 0; q < round; ++q) in = in && bucket_of(d, q) == pick[q];
         const int bk = bucket_of(d, round);
         if (in && bk >= 0) cols[bk * SMP_THREADS + tid] += e;
-      }
+      });
       // bucket sums: wave sums, then sixteen threads add the waves' partial sums
       for (int b = 0; b < SMP_FAN; ++b) {
         const float v = wave_sum(cols[b * SMP_THREADS + tid]);
@@ -221,8 +257,7 @@ sample_top_p_kernel(int32_t* __restrict__ out, float* __restrict__ work, int wan
       width *= 1.0f / SMP_FAN;
     }
     if (found) {
-      for (int i = tid; i < V; i += SMP_THREADS) {
-        const float e = ex[i];
+      for_row(ex, V, vec_ex, [&](int, float e) {
         const float d = fmaxf(-__builtin_amdgcn_logf(e) * 0.6931471805599453f, 0.f);   // e may be a hair above 1
         bool in = true;
 #pragma unroll
@@ -231,7 +266,7 @@ sample_top_p_kernel(int32_t* __restrict__ out, float* __restrict__ work, int wan
           const int at = atomicAdd(&list_n, 1);
           if (at < SMP_LIST) list[at] = e;
         }
-      }
+      });
       __syncthreads();
       const int n = list_n;
       // lo keeps mass_above(lo) > top_p, hi keeps mass_above(hi) <= top_p
