@@ -13,9 +13,9 @@
 // A workgroup of four waves takes 64 or 128 query rows of one head (16 or 32 per
 // wave) and walks the sequence's keys in tiles of 64. Key and value tiles go
 // through LDS as they lie in the cache (rows of D), in two buffers: while tile t
-// is used, tile t+1 is written to the other buffer from registers and tile t+2 is
-// on its way from global memory into those registers (its page numbers were read
-// one tile earlier still), so a tile costs one barrier. Both products are
+// is used, tile t+1 is on its way from global memory straight into the other
+// buffer (global_load_lds_dwordx4, no register in between; its page numbers were
+// read one tile earlier still), so a tile costs one barrier. Both products are
 // computed transposed so that the scores leave the first MFMA in the register
 // layout the second one wants, without a shuffle:
 //   S^T[key, query] = K[key, :] . Q[query, :]      (A = K tile, B = Q^T)
@@ -59,29 +59,41 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ q_start,
                          const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ block_table,
                          int bt_stride, const int32_t* __restrict__ work_seq,
-                         const int32_t* __restrict__ work_qoff, int Hq, int Hkv, int page_size,
-                         int page_shift, int window, float scale_log2) {
+                         const int32_t* __restrict__ work_qoff, int n_work, int Hq, int Hkv,
+                         int page_size, int page_shift, int window, float scale_log2) {
   constexpr int D = 32 * NDT;
   constexpr int PBM = 64 * RT;
-  constexpr int KS = D + 8;            // row stride of the key tile, in elements
-  constexpr int VS = D + 16;           // row stride of the value tile
   constexpr int CPR = D / 8;           // 16-byte chunks per row
   constexpr int NCH = PF_BN * CPR / 256;   // chunks of a tile per thread
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[2][PF_BN * KS];
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[2][PF_BN * VS];
+  // Tiles lie in LDS as rows of D elements without padding; the 16-byte chunks of a row are
+  // permuted (chunk c of row r lies at c ^ swz(r)) so that neither the row-wise reads of the
+  // first product nor the transposing reads of the second meet in a bank. Two buffers each,
+  // as separate arrays: the compiler then knows that a load into one does not touch the other.
+  constexpr bool SW8 = CPR % 8 == 0;
+  __shared__ __attribute__((aligned(1024))) bf16_t Ks0[PF_BN * D];
+  __shared__ __attribute__((aligned(1024))) bf16_t Ks1[PF_BN * D];
+  __shared__ __attribute__((aligned(1024))) bf16_t Vs0[PF_BN * D];
+  __shared__ __attribute__((aligned(1024))) bf16_t Vs1[PF_BN * D];
+  auto swz = [](int row) { return SW8 ? (row & 7) : ((row >> 1) & 3); };
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 15, lg = lane >> 4;
   const int xor16 = 4 * (lane ^ 16), xor32 = 4 * (lane ^ 32);
   const int head = blockIdx.y;
-  const int seq = work_seq[blockIdx.x];
-  const int qoff = work_qoff[blockIdx.x];
+  // The work list is sorted, the blocks with the most keys first. The gridDim.x workgroups of a
+  // head walk it as a snake: forwards in even rounds, backwards in odd ones, so that the
+  // workgroup with the longest block of one round takes the shortest of the next.
+  for (int round = 0;; ++round) {
+  const int item = round * gridDim.x + ((round & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
+  if (item >= n_work) break;       // (and so is every later item of this workgroup)
+  const int seq = work_seq[item];
+  const int qoff = work_qoff[item];
   const int qs = q_start[seq];
   const int qlen = q_start[seq + 1] - qs;
   const int ctx = ctx_len[seq];
   const int cached = ctx - qlen;
   const int rows = min(PBM, qlen - qoff);
-  if (rows <= 0) return;
+  if (rows <= 0) continue;
   const int kvh = head / (Hq / Hkv);
   const int32_t* bt = block_table + (size_t)seq * bt_stride;
   const int first_q = cached + qoff;
@@ -105,17 +117,14 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
   const int wave_min_q = first_q + (wave_has_rows ? wave_first_row : 0);
   const int wave_max_q = first_q + min(rows, wave_first_row + 16 * RT) - 1;
 
-  // The softmax denominator. 16 rows a wave (registers to spare): o[r][2 NDT] is one more tile
-  // of the second product, whose "values" are all one; it sums the probabilities as the product
-  // sees them (rounded to bfloat16; float32 sums) and is rescaled with the numerators. 32 rows
-  // a wave: every lane adds its probabilities (float32) and the lanes of a column meet at the end.
-  constexpr bool L_MFMA = RT == 1;
+  // The softmax denominator: o[r][2 NDT] is one more tile of the second product, whose
+  // "values" are all one; it sums the probabilities as the product sees them (rounded to
+  // bfloat16; float32 sums) and is rescaled with the numerators.
   f32x4_t o[RT][2 * NDT + 1];
-  float m_run[RT], l_part[RT];
+  float m_run[RT];
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
     m_run[r] = -INFINITY;
-    l_part[r] = 0.f;
 #pragma unroll
     for (int t = 0; t <= 2 * NDT; ++t) o[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
@@ -132,19 +141,20 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
   const int k_begin = (k_lo / PF_BN) * PF_BN;
   const int n_tiles = (k_end - k_begin + PF_BN - 1) / PF_BN;
 
-  // this thread's chunks of a tile: key row crow[i], elements ccol[i] .. +7
+  // This thread's chunks of a tile. A wave's load instruction fills 64 consecutive 16-byte
+  // slots of LDS, lane l the l-th; slot s holds row s / CPR, chunk (s % CPR) ^ swz(row).
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   int crow[NCH], ccol[NCH];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = tid + 256 * i;
-    crow[i] = c / CPR;
-    ccol[i] = (c - crow[i] * CPR) * 8;
+    const int slot = 64 * (wave_u * NCH + i) + lane;
+    crow[i] = slot / CPR;
+    ccol[i] = ((slot - crow[i] * CPR) ^ swz(crow[i])) * 8;
   }
   const bf16_t* k_head = k_cache + (size_t)kvh * page_size * D;
   const bf16_t* v_head = v_cache + (size_t)kvh * page_size * D;
 
   int pg[NCH];                  // pages of the chunks' rows, read one tile ahead of the rows
-  uint4 kreg[NCH], vreg[NCH];   // carry a tile from global memory to LDS
   const uint32_t page_bytes = (uint32_t)Hkv * page_size * D * 2;     // < 4 GiB, checked by the host
   const int page_mask = page_size - 1;                                // page sizes are powers of two
   // a tile that lies wholly inside the keys this block sees needs no tests (uniform)
@@ -166,37 +176,52 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
       }
     }
   };
-  auto issue_loads = [&](int t) {
+  // global memory -> LDS without a register in between (global_load_lds_dwordx4): every lane
+  // names its own 16 bytes of global memory, the wave's 64 chunks land side by side in LDS
+  auto to_lds = [&](const bf16_t* base, uint64_t at, bf16_t* tile_lds, int i) {
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)(reinterpret_cast<const char*>(base) + at),
+        (__attribute__((address_space(3))) void*)(tile_lds + 512 * (wave_u * NCH + i)), 16, 0, 0);
+  };
+  auto fetch = [&](int t, bf16_t* Kb, bf16_t* Vb) {
     const int k0 = k_begin + t * PF_BN;
     if (whole(t)) {
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
         const uint32_t in_page = (uint32_t)(((k0 + crow[i]) & page_mask) * D + ccol[i]) * 2;
         const uint64_t at = (uint64_t)(uint32_t)pg[i] * page_bytes + in_page;
-        kreg[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(k_head) + at);
-        vreg[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(v_head) + at);
+        to_lds(k_head, at, Kb, i);
+        to_lds(v_head, at, Vb, i);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
-        kreg[i] = make_uint4(0, 0, 0, 0);       // rows outside the keys read as zeros
-        vreg[i] = make_uint4(0, 0, 0, 0);
         if (pg[i] >= 0) {
           const uint32_t in_page = (uint32_t)(((k0 + crow[i]) & page_mask) * D + ccol[i]) * 2;
           const uint64_t at = (uint64_t)(uint32_t)pg[i] * page_bytes + in_page;
-          kreg[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(k_head) + at);
-          vreg[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(v_head) + at);
+          to_lds(k_head, at, Kb, i);
+          to_lds(v_head, at, Vb, i);
+        } else {                                  // rows outside the keys read as zeros
+          const int slot = 64 * (wave_u * NCH + i) + lane;
+          *reinterpret_cast<uint4*>(Kb + 8 * slot) = make_uint4(0, 0, 0, 0);
+          *reinterpret_cast<uint4*>(Vb + 8 * slot) = make_uint4(0, 0, 0, 0);
         }
       }
     }
   };
-  auto write_lds = [&](int b) {
+  // where this lane reads: the first product takes row 16 kt + ln, chunk 4 kk + lg; the second
+  // points at row 32 half + 16 j + 4 lg + ln / 4, elements 16 dt + 4 (ln % 4) .. +3
+  int k_at[NDT], v_at[2 * NDT];
+  {
+    const int sw = swz(ln);
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      *reinterpret_cast<uint4*>(&Ks[b][crow[i] * KS + ccol[i]]) = kreg[i];
-      *reinterpret_cast<uint4*>(&Vs[b][crow[i] * VS + ccol[i]]) = vreg[i];
-    }
-  };
+    for (int kk = 0; kk < NDT; ++kk) k_at[kk] = ln * D + 8 * ((4 * kk + lg) ^ sw);
+    const int vrow = 4 * lg + (ln >> 2);
+    const int vsw = swz(vrow);
+#pragma unroll
+    for (int dt = 0; dt < 2 * NDT; ++dt)
+      v_at[dt] = vrow * D + 8 * ((2 * dt + ((ln & 3) >> 1)) ^ vsw) + 4 * (ln & 1);
+  }
 
   // one key tile for this wave's rows; MASKED: the tile touches the diagonal, the end of the
   // keys or a window's edge
@@ -210,7 +235,7 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
 #pragma unroll
       for (int kk = 0; kk < NDT; ++kk) {
         Frag8 a;
-        a.u = *reinterpret_cast<const uint4*>(Kb + (16 * kt + ln) * KS + 32 * kk + 8 * lg);
+        a.u = *reinterpret_cast<const uint4*>(Kb + 16 * kt * D + k_at[kk]);
 #pragma unroll
         for (int r = 0; r < RT; ++r)
           st[r][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[r][kk].v, st[r][kt], 0, 0, 0);
@@ -244,9 +269,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
       if (tmax > m_run[r] + lazy) {
         const float alpha = __builtin_amdgcn_exp2f((m_run[r] - tmax) * scale_log2);
         m_run[r] = tmax;
-        l_part[r] *= alpha;
 #pragma unroll
-        for (int t = 0; t < 2 * NDT + (L_MFMA ? 1 : 0); ++t) {
+        for (int t = 0; t <= 2 * NDT; ++t) {
           o[r][t][0] *= alpha; o[r][t][1] *= alpha; o[r][t][2] *= alpha; o[r][t][3] *= alpha;
         }
       }
@@ -259,65 +283,61 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const float p = __builtin_amdgcn_exp2f(fmaf(st[r][2 * half + t][i], scale_log2, mc));
-            if (!L_MFMA) l_part[r] += p;
             pb[r][half].v[4 * t + i] = (__bf16)p;
           }
     }
     // V^T fragments: lane (ln, lg) points at V[key0 + ln/4][16 dt + 4 (ln%4)] and receives
     // V[key0 + 0..3][16 dt + ln], key0 = 32 half + 16 t + 4 lg: the keys of P^T's element 4 t + i
-    const bf16_t* vp = Vb + (4 * lg + (ln >> 2)) * VS + 4 * (ln & 3);
 #pragma unroll
     for (int half = 0; half < 2; ++half)
 #pragma unroll
       for (int dt = 0; dt < 2 * NDT; ++dt) {
         Frag8 a;
-        a.s[0] = lds_read_tr16(vp + (32 * half) * VS + 16 * dt);
-        a.s[1] = lds_read_tr16(vp + (32 * half + 16) * VS + 16 * dt);
+        a.s[0] = lds_read_tr16(Vb + (32 * half) * D + v_at[dt]);
+        a.s[1] = lds_read_tr16(Vb + (32 * half + 16) * D + v_at[dt]);
 #pragma unroll
         for (int r = 0; r < RT; ++r)
           o[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb[r][half].v, o[r][dt], 0, 0, 0);
       }
-    if (L_MFMA) {
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
+    for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int r = 0; r < RT; ++r)
-          o[r][2 * NDT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[r][half].v, o[r][2 * NDT], 0, 0, 0);
-    }
+      for (int r = 0; r < RT; ++r)
+        o[r][2 * NDT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[r][half].v, o[r][2 * NDT], 0, 0, 0);
   };
 
-  load_pages(0);
-  issue_loads(0);
-  load_pages(1);
-  write_lds(0);
-  issue_loads(1);
-  load_pages(2);
-  __syncthreads();
-  for (int t = 0; t < n_tiles; ++t) {
+  // one turn: tile t + 1 sets out for the other buffer (everyone left it before the last
+  // barrier), tile t is used, and what was loaded is waited for before the barrier
+  auto turn = [&](int t, bf16_t* Kb, bf16_t* Vb, bf16_t* Kn, bf16_t* Vn) {
     const int k0 = k_begin + t * PF_BN;
     if (t + 1 < n_tiles) {
-      write_lds((t + 1) & 1);           // everyone left that buffer before the last barrier
-      issue_loads(t + 2);
-      load_pages(t + 3);
+      fetch(t + 1, Kn, Vn);
+      load_pages(t + 2);
     }
     // a wave whose rows all lie before this tile has nothing to do in it
     if (wave_has_rows && k0 <= wave_max_q) {
       const bool need_mask = (k0 + PF_BN - 1 > wave_min_q) || (k0 + PF_BN > k_end) || window > 0;
       if (need_mask)
-        tile(k0, Ks[t & 1], Vs[t & 1], std::true_type{});
+        tile(k0, Kb, Vb, std::true_type{});
       else
-        tile(k0, Ks[t & 1], Vs[t & 1], std::false_type{});
+        tile(k0, Kb, Vb, std::false_type{});
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this wave's loads into LDS have landed
     __syncthreads();
+  };
+  load_pages(0);
+  fetch(0, Ks0, Vs0);
+  load_pages(1);
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  for (int t = 0; t < n_tiles; t += 2) {
+    turn(t, Ks0, Vs0, Ks1, Vs1);
+    if (t + 1 < n_tiles) turn(t + 1, Ks1, Vs1, Ks0, Vs0);
   }
 
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
-    float l = o[r][2 * NDT][0];                // every row of that tile holds the column's sum
-    if (!L_MFMA) {
-      l = l_part[r] + __shfl_xor(l_part[r], 16, 64);
-      l += __shfl_xor(l, 32, 64);
-    }
+    const float l = o[r][2 * NDT][0];          // every row of that tile holds the column's sum
     if (row_ok[r]) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;
       const int my_row = 16 * (RT * wave + r) + ln;
@@ -331,26 +351,29 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
       }
     }
   }
+  }   // work items
 }
 
 template <int NDT, int RT>
 static int launch_prefill_mfma(void* out, long out_stride, const void* q, long q_stride,
                                const void* k_cache, const void* v_cache, const int32_t* q_start,
                                const int32_t* ctx_len, const int32_t* block_table, int bt_stride,
-                               const int32_t* work_seq, const int32_t* work_qoff, int n_work, int Hq,
-                               int Hkv, int page_size, int window, float scale, hipStream_t stream) {
-  dim3 grid(n_work, Hq);
+                               const int32_t* work_seq, const int32_t* work_qoff, int n_work,
+                               int n_groups, int Hq, int Hkv, int page_size, int window, float scale,
+                               hipStream_t stream) {
+  dim3 grid(n_groups, Hq);
   int page_shift = -1;
   for (int sh = 0; sh < 31; ++sh)
     if ((1 << sh) == page_size) page_shift = sh;
   attn_prefill_mfma_kernel<NDT, RT><<<grid, 256, 0, stream>>>(
       (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-      (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff, Hq, Hkv,
-      page_size, page_shift, window, scale * 1.4426950408889634f);
+      (const bf16_t*)v_cache, q_start, ctx_len, block_table, bt_stride, work_seq, work_qoff,
+      n_work, Hq, Hkv, page_size, page_shift, window, scale * 1.4426950408889634f);
   return ptl_launch_status();
 }
 
-// work_seq / work_qoff list query blocks of ``block_rows`` rows (64 or 128). bfloat16 only;
+// work_seq / work_qoff list query blocks of ``block_rows`` rows (64 or 128), the longest first;
+// n_groups workgroups a head share them (1 <= n_groups <= n_work). bfloat16 only;
 // q rows must be 16-byte aligned and output rows 8-byte (q_stride % 8, out_stride % 4); the
 // page size is a power of two and a page of all kv heads is smaller than 4 GiB.
 extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void* q, long q_stride,
@@ -358,17 +381,19 @@ extern "C" int ptl_attention_prefill_mfma(void* out, long out_stride, const void
                                           const int32_t* q_start, const int32_t* ctx_len,
                                           const int32_t* block_table, int bt_stride,
                                           const int32_t* work_seq, const int32_t* work_qoff,
-                                          int n_work, int block_rows, int Hq, int Hkv, int D,
+                                          int n_work, int n_groups, int block_rows, int Hq,
+                                          int Hkv, int D,
                                           int page_size, int window, float scale,
                                           hipStream_t stream) {
   if (n_work <= 0) return PTL_OK;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || D % 32 || D <= 0 || D > 128 || page_size <= 0 ||
       (page_size & (page_size - 1)) || (long)Hkv * page_size * D * 2 >= (1L << 32) ||
-      Hq > 65535 || q_stride % 8 || out_stride % 4 || (block_rows != 64 && block_rows != 128))
+      Hq > 65535 || n_groups < 1 || n_groups > n_work || q_stride % 8 || out_stride % 4 ||
+      (block_rows != 64 && block_rows != 128))
     return PTL_ERR_ARG;
 #define GO(N, R) launch_prefill_mfma<N, R>(out, out_stride, q, q_stride, k_cache, v_cache, q_start, \
                                            ctx_len, block_table, bt_stride, work_seq, work_qoff,  \
-                                           n_work, Hq, Hkv, page_size, window, scale, stream)
+                                           n_work, n_groups, Hq, Hkv, page_size, window, scale, stream)
   if (block_rows == 64) {
     switch (D / 32) {
       case 1: return GO(1, 1);

@@ -7,6 +7,7 @@ raises.
 from __future__ import annotations
 
 import ctypes
+import functools
 from typing import Optional
 
 import torch
@@ -482,13 +483,35 @@ def attention_prefill_mfma_fits(dtype: torch.dtype, num_kv_heads: int, head_dim:
             and num_kv_heads * page_size * head_dim * 2 < 2 ** 32)
 
 
+@functools.lru_cache(maxsize=None)
+def _compute_units(device_index: int) -> int:
+    return int(torch.cuda.get_device_properties(device_index).multi_processor_count)
+
+
+def attention_prefill_mfma_plan(device: torch.device, num_heads: int, head_dim: int,
+                                blocks_of_64: int, blocks_of_128: int):
+    """(block_rows, groups) for ``attention_prefill_mfma``. As many workgroups a head as the
+    chip holds at once (three a compute unit up to head size 64, two above), so that all run
+    side by side and the snake over the sorted work list evens out the causal triangle;
+    128-row blocks (keys and values are staged half as often) only when every workgroup gets
+    at least two of them."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    resident = _compute_units(index) * (3 if head_dim <= 64 else 2)
+    groups = max(1, resident // num_heads)
+    if blocks_of_128 >= 2 * groups:
+        return 128, groups
+    return 64, max(1, min(groups, blocks_of_64))
+
+
 def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                            v_cache: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                            block_table: torch.Tensor, work_seq: torch.Tensor,
                            work_qoff: torch.Tensor, scale: float, window: int = 0,
-                           block_rows: int = 64) -> None:
+                           block_rows: int = 64, groups: int = 0) -> None:
     """bfloat16 attention of prompt portions on the matrix cores; the work list
-    names query blocks of ``block_rows`` (64 or 128) rows. Head sizes 32, 64, 96, 128."""
+    names query blocks of ``block_rows`` (64 or 128) rows, those with the most
+    keys first. ``groups`` workgroups a head share the list (0: one for every
+    block). Head sizes 32, 64, 96, 128."""
     T, Hq, Hkv, D, page_size = _attention_common(out, q, k_cache, v_cache, q_start, ctx_len,
                                                  block_table, "attention_prefill_mfma")
     if q.dtype != torch.bfloat16:
@@ -508,12 +531,13 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
     if q.stride(0) % 8 or out.stride(0) % 4 or q.data_ptr() % 16 or out.data_ptr() % 8:
         raise KernelError("attention_prefill_mfma: q rows must be 16-byte aligned, out rows 8-byte")
     lib = library.load("attention_prefill")
+    n_work = int(work_seq.numel())
     _check(lib.ptl_attention_prefill_mfma(
         _ptr(out), ctypes.c_long(out.stride(0)), _ptr(q), ctypes.c_long(q.stride(0)),
         _ptr(k_cache), _ptr(v_cache), _ptr(q_start), _ptr(ctx_len), _ptr(block_table),
-        int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), int(work_seq.numel()),
-        int(block_rows), Hq, Hkv, D, page_size, int(window), ctypes.c_float(scale), _stream()),
-        "attention_prefill_mfma")
+        int(block_table.stride(0)), _ptr(work_seq), _ptr(work_qoff), n_work,
+        min(n_work, int(groups)) if groups > 0 else n_work, int(block_rows), Hq, Hkv, D, page_size,
+        int(window), ctypes.c_float(scale), _stream()), "attention_prefill_mfma")
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

@@ -153,11 +153,12 @@ class PagedAttention(Part):
             return
         if (ops.attention_prefill_mfma_fits(q.dtype, self.num_kv_heads, D, cache.page_size)
                 and q.stride(0) % 8 == 0):
-            # long portions in 128-row blocks (keys and values are staged half as often)
-            rows = 128 if ctx.max_q_len >= 256 and D <= 64 else 64
+            rows, groups = ops.attention_prefill_mfma_plan(
+                q.device, self.num_heads, D, ctx.work["multi64"][0].numel(),
+                ctx.work["multi128"][0].numel())
             ws, wo = ctx.work["multi128" if rows == 128 else "multi64"]
             ops.attention_prefill_mfma(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
-                                       group.block_table, ws, wo, self.scale, window, rows)
+                                       group.block_table, ws, wo, self.scale, window, rows, groups)
         else:
             ws, wo = ctx.work["multi16"] if n_dec else ctx.work["all16"]
             ops.attention_generic(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,

@@ -298,7 +298,7 @@ def _paged_setup(seq_lens, q_lens, Hkv, D, P, dtype, seed, shuffle=True):
 
 
 def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=0, boost=None,
-                    kernel="generic", splits=1, unroll=0):
+                    kernel="generic", splits=1, unroll=0, groups=0):
     kc, vc, bt, dk, dv = _paged_setup(seq_lens, q_lens, Hkv, D, P, dtype, seed)
     g = torch.Generator().manual_seed(seed + 100)
     T = sum(q_lens)
@@ -327,7 +327,8 @@ def _attention_case(ops, dtype, seq_lens, q_lens, Hq, Hkv, D, P, window=0, seed=
                               bt.to(dev), i32(work_seq), i32(work_qoff), scale, window)
     elif kernel in ("mfma", "mfma128"):
         ops.attention_prefill_mfma(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
-                                   bt.to(dev), i32(work_seq), i32(work_qoff), scale, window, rows)
+                                   bt.to(dev), i32(work_seq), i32(work_qoff), scale, window, rows,
+                                   groups)
     else:
         assert all(ql == 1 for ql in q_lens)
         ops.attention_decode(out, qd, kc.to(dev), vc.to(dev), i32(q_start), i32(seq_lens),
@@ -430,6 +431,29 @@ def test_attention_prefill_mfma_refuses_odd_page_size(ops):
     with pytest.raises(ops.KernelError, match="power of two"):
         _attention_case(ops, torch.bfloat16, seq_lens=[150], q_lens=[70], Hq=2, Hkv=1, D=32, P=5,
                         kernel="mfma")
+
+
+@pytest.mark.parametrize("groups", [1, 2, 3, 5])
+@pytest.mark.parametrize("kernel", ["mfma", "mfma128"])
+def test_attention_prefill_mfma_workgroups_share_the_blocks(ops, kernel, groups):
+    """Fewer workgroups a head than query blocks: each walks several blocks (of different
+    sequences, with and without a prefix in the cache), forwards and backwards over the
+    list, and reuses its LDS buffers from one block to the next."""
+    _attention_case(ops, torch.bfloat16, seq_lens=[520, 90, 300], q_lens=[390, 90, 129], Hq=4, Hkv=2,
+                    D=64, P=16, kernel=kernel, groups=groups)
+    _attention_case(ops, torch.bfloat16, seq_lens=[333], q_lens=[333], Hq=2, Hkv=1, D=128, P=8,
+                    window=100, kernel=kernel, groups=groups)
+
+
+def test_attention_prefill_mfma_plan(ops):
+    """128-row blocks only when every workgroup gets two; never more workgroups than blocks."""
+    dev = torch.device("cuda", 0)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    per_head = max(1, 3 * cus // 32)
+    assert ops.attention_prefill_mfma_plan(dev, 32, 64, 3, 2) == (64, min(3, per_head))
+    assert ops.attention_prefill_mfma_plan(dev, 32, 64, 4 * per_head, 2 * per_head) == (128, per_head)
+    assert ops.attention_prefill_mfma_plan(dev, 32, 64, 4 * per_head - 2, 2 * per_head - 1) == (64, per_head)
+    assert ops.attention_prefill_mfma_plan(dev, 4 * cus, 128, 1, 1) == (64, 1)
 
 
 def test_attention_prefill_mfma_long(ops):
