@@ -19,6 +19,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 from ..parts.base import PagedKVSpec, StateSpec
 
 RELEASED = -1   # block-table entry of a page that was given back (left of the window)
@@ -181,17 +183,23 @@ class CacheManager:
         self.num_tokens[req] = start + n_new
         return start
 
-    def slots(self, req, group: int, start: int, n: int) -> List[int]:
-        """Flat cache slots page*page_size+offset of positions start..start+n-1."""
+    def slot_array(self, req, group: int, start: int, n: int) -> np.ndarray:
+        """Flat cache slots page*page_size+offset of positions start..start+n-1 (int32)."""
         table = self.paged[group].tables[req]
         P = self.page_size
-        out = []
-        for pos in range(start, start + n):
-            page = table[pos // P]
-            if page < 0:
-                raise RuntimeError(f"request {req!r}: position {pos} lies in a released page")
-            out.append(page * P + pos % P)
-        return out
+        first = start // P
+        pages = np.asarray(table[first:(start + n - 1) // P + 1], dtype=np.int64)
+        if n <= 0 or pages.size != (start + n - 1) // P + 1 - first:
+            raise RuntimeError(f"request {req!r}: positions {start}..{start + n - 1} lie outside its pages")
+        if (pages < 0).any():
+            pos = (first + int(np.argmax(pages < 0))) * P
+            raise RuntimeError(f"request {req!r}: position {max(pos, start)} lies in a released page")
+        pos = np.arange(start, start + n, dtype=np.int64)
+        return (pages[pos // P - first] * P + pos % P).astype(np.int32)
+
+    def slots(self, req, group: int, start: int, n: int) -> List[int]:
+        """The same as a list."""
+        return self.slot_array(req, group, start, n).tolist()
 
     def release_behind_window(self, req) -> int:
         """Give back the pages of ``req`` that no later query can read (groups

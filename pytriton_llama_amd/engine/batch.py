@@ -12,6 +12,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 GENERIC_BLOCK_ROWS = 16   # query rows per work item of the vector-FMA attention kernel
@@ -22,14 +23,18 @@ MFMA_BIG_BLOCK_ROWS = 128  # ... and for long ones
 def work_items(q_lens, ctx_lens, first_seq: int, block_rows: int):
     """(sequence, first row) of every block of ``block_rows`` query rows of the
     sequences from ``first_seq`` on, the blocks with the most keys first so
-    that the long ones do not end the launch alone."""
-    items = []
+    that the long ones do not end the launch alone. Two int32 arrays."""
+    seqs, offs, keys = [], [], []
     for s in range(first_seq, len(q_lens)):
-        cached = ctx_lens[s] - q_lens[s]
-        for off in range(0, q_lens[s], block_rows):
-            items.append((cached + min(off + block_rows, q_lens[s]), s, off))
-    items.sort(key=lambda t: -t[0])
-    return [s for _, s, _ in items], [o for _, _, o in items]
+        off = np.arange(0, q_lens[s], block_rows, dtype=np.int32)
+        seqs.append(np.full(off.size, s, dtype=np.int32))
+        offs.append(off)
+        keys.append(ctx_lens[s] - q_lens[s] + np.minimum(off + block_rows, q_lens[s]))
+    if not seqs:
+        return np.zeros(0, dtype=np.int32), np.zeros(0, dtype=np.int32)
+    seqs, offs, keys = np.concatenate(seqs), np.concatenate(offs), np.concatenate(keys)
+    by_keys = np.argsort(-keys, kind="stable")
+    return seqs[by_keys], offs[by_keys]
 
 
 @dataclass
@@ -79,9 +84,11 @@ def order_entries(entries: Sequence[StepEntry]) -> List[int]:
            [i for i in idx if len(entries[i].tokens) != 1]
 
 
-def take_pages(entries: Sequence[StepEntry], manager, vocab_size: Optional[int] = None) -> List[int]:
+def take_pages(entries: Sequence[StepEntry], manager, vocab_size: Optional[int] = None,
+               token_arrays: Optional[list] = None) -> List[int]:
     """Check the entries and take the pages for all of them, or for none.
-    Returns the position of every entry's first token."""
+    Returns the position of every entry's first token. ``token_arrays``: a list
+    that receives every entry's tokens as an int32 array."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     seen = set()
@@ -95,11 +102,16 @@ def take_pages(entries: Sequence[StepEntry], manager, vocab_size: Optional[int] 
             if not 0 <= w < len(e.tokens):
                 raise ValueError(f"request {e.request!r}: wanted place {w} outside its "
                                  f"{len(e.tokens)} tokens")
-        if vocab_size is not None:
-            for t in e.tokens:
-                if not 0 <= t < vocab_size:
-                    raise ValueError(f"request {e.request!r}: token id {t} outside the "
-                                     f"vocabulary of {vocab_size}")
+        if len(e.tokens) == 1 and token_arrays is None:
+            bad = [] if vocab_size is None or 0 <= e.tokens[0] < vocab_size else [e.tokens[0]]
+        else:
+            toks = np.asarray(e.tokens)
+            bad = toks[(toks < 0) | (toks >= vocab_size)] if vocab_size is not None else []
+            if token_arrays is not None:
+                token_arrays.append(toks.astype(np.int32, copy=False))
+        if len(bad):
+            raise ValueError(f"request {e.request!r}: token id {int(bad[0])} outside the "
+                             f"vocabulary of {vocab_size}")
     need = [0] * len(manager.paged)
     for e in entries:
         for g, n in enumerate(manager.pages_needed(e.request, len(e.tokens))):
@@ -116,30 +128,31 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
     """Take pages for every entry (all or nothing) and lay the batch out.
     Returns (StepContext, order) where ``order`` is the permutation applied to
     the entries; logit rows are listed in the caller's order of entries."""
-    starts = take_pages(entries, manager, vocab_size)
+    tokens_of: list = []
+    starts = take_pages(entries, manager, vocab_size, tokens_of)
 
     order = order_entries(entries)
-    token_ids: List[int] = []
-    positions: List[int] = []
+    i32 = lambda values: np.asarray(values, dtype=np.int32)
+    token_ids, positions = [], []
     q_start = [0]
     ctx_len: List[int] = []
     state_slots: List[int] = []
-    slots: List[List[int]] = [[] for _ in manager.paged]
+    slots: List[list] = [[] for _ in manager.paged]
     row_of_entry = {}
     for i in order:
         e = entries[i]
         n = len(e.tokens)
         start = starts[i]
         row_of_entry[i] = q_start[-1]
-        token_ids.extend(int(t) for t in e.tokens)
-        positions.extend(range(start, start + n))
+        token_ids.append(tokens_of[i])
+        positions.append(np.arange(start, start + n, dtype=np.int32))
         q_start.append(q_start[-1] + n)
         ctx_len.append(start + n)
         state_slots.append(manager.slot_of[e.request])
         for g in range(len(manager.paged)):
-            slots[g].extend(manager.slots(e.request, g, start, n))
+            slots[g].append(manager.slot_array(e.request, g, start, n))
     logit_rows = [row_of_entry[i] + w for i, e in enumerate(entries) for w in e.want]
-    T = len(token_ids)
+    T = q_start[-1]
     nseq = len(order)
     q_lens = [q_start[i + 1] - q_start[i] for i in range(nseq)]
     num_decode = 0
@@ -153,18 +166,25 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
     for g, group in enumerate(manager.paged):
         rows = [group.tables[entries[i].request] for i in order]
         width = max(1, max(len(r) for r in rows))
-        tables.append([r + [-1] * (width - len(r)) for r in rows])
+        table = np.full((nseq, width), -1, dtype=np.int32)
+        for r, row in enumerate(rows):
+            table[r, :len(row)] = row
+        tables.append(table)
 
     # one host->device copy for all integer arrays
-    flat: List[int] = []
+    parts: List[np.ndarray] = []
     spans = {}
+    filled = 0
 
     def put(name, values):
-        spans[name] = (len(flat), len(values))
-        flat.extend(values)
+        nonlocal filled
+        values = i32(values).reshape(-1)
+        spans[name] = (filled, values.size)
+        parts.append(values)
+        filled += values.size
 
-    put("token_ids", token_ids)
-    put("positions", positions)
+    put("token_ids", np.concatenate(token_ids))
+    put("positions", np.concatenate(positions))
     put("q_start", q_start)
     put("ctx_len", ctx_len)
     put("state_slots", state_slots)
@@ -173,11 +193,14 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
         put("ws_" + name, ws)
         put("wo_" + name, wo)
     for g in range(len(manager.paged)):
-        put(f"slots{g}", slots[g])
-        put(f"table{g}", [p for row in tables[g] for p in row])
-    buf = torch.tensor(flat, dtype=torch.int32)
+        put(f"slots{g}", np.concatenate(slots[g]))
+        put(f"table{g}", tables[g])
     if torch.device(device).type != "cpu":
-        buf = buf.pin_memory().to(device, non_blocking=True)
+        staged = torch.empty(filled, dtype=torch.int32, pin_memory=True)
+        np.concatenate(parts, out=staged.numpy())
+        buf = staged.to(device, non_blocking=True)
+    else:
+        buf = torch.from_numpy(np.concatenate(parts))
 
     def get(name):
         a, n = spans[name]
@@ -190,7 +213,7 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: Opt
         ctx_len=get("ctx_len"), state_slots=get("state_slots"), logit_rows=get("logit_rows"),
         work={name: (get("ws_" + name), get("wo_" + name)) for name in work}, groups=groups,
         num_tokens=T, num_seqs=nseq, num_logit_rows=len(logit_rows),
-        logit_rows_are_identity=logit_rows == list(range(T)),
+        logit_rows_are_identity=len(logit_rows) == T and logit_rows == list(range(T)),
         num_decode_seqs=num_decode,
         q_lens=q_lens, ctx_lens=ctx_len, max_q_len=max(q_lens), max_ctx_len=max(ctx_len))
     return ctx, order

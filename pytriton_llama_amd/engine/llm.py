@@ -5,6 +5,7 @@ import itertools
 import os
 from typing import Dict, Hashable, Iterator, List, Optional, Sequence, Union
 
+import numpy as np
 import torch
 
 from ..cache import CacheManager, CacheStorage
@@ -93,10 +94,13 @@ class Engine:
         if rid in self.requests:
             raise ValueError(f"request id {rid!r} is in use")
         V = self.model.vocab_size
-        for t in prompt:
-            if not 0 <= int(t) < V:
-                raise ValueError(f"token id {t} outside the vocabulary of {V}")
-        req = Request(rid, [int(t) for t in prompt], params or SamplingParams())
+        ids = np.asarray(prompt if not isinstance(prompt, torch.Tensor) else prompt.cpu())
+        if ids.ndim != 1 or (ids.size and ids.dtype.kind not in "iu"):
+            raise ValueError("a prompt is a sequence of token ids (integers)")
+        outside = ids[(ids < 0) | (ids >= V)]
+        if outside.size:
+            raise ValueError(f"token id {int(outside[0])} outside the vocabulary of {V}")
+        req = Request(rid, ids.astype(np.int32), params or SamplingParams())
         self.scheduler.add(req)
         self.requests[rid] = req
         return rid

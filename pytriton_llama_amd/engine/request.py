@@ -4,6 +4,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional
 
+import numpy as np
+
 
 @dataclass
 class SamplingParams:
@@ -42,15 +44,22 @@ class Request:
     finish_reason: Optional[str] = None
     num_preemptions: int = 0
 
+    def __post_init__(self):
+        # the prompt as a list and as an array: portions of it go to the step without a conversion
+        self.prompt_array = np.asarray(self.prompt, dtype=np.int32).reshape(-1)
+        if not isinstance(self.prompt, list):
+            self.prompt = self.prompt_array.tolist()
+
     @property
     def tokens(self) -> List[int]:
         return self.prompt + self.output
 
-    def token_slice(self, start: int, n: int) -> List[int]:
-        """tokens[start:start+n] without joining prompt and output."""
+    def token_slice(self, start: int, n: int):
+        """tokens[start:start+n] without joining prompt and output (a portion of the prompt
+        as an int32 array, anything else as a list)."""
         np_ = len(self.prompt)
         if start + n <= np_:
-            return self.prompt[start:start + n]
+            return self.prompt_array[start:start + n] if n > 1 else self.prompt[start:start + n]
         if start >= np_:
             return self.output[start - np_:start - np_ + n]
         return self.prompt[start:] + self.output[:start + n - np_]
