@@ -334,15 +334,6 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   __shared__ float row_factor[16];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, lg = lane >> 4;
   const int nwaves = blockDim.x >> 6;
-  if (sc.partials != nullptr) {
-    // the waves share the rows; a row's partial sums are added in a fixed order
-    for (int m = wave; m < M; m += nwaves) {
-      float sum = 0.f;
-      for (int j = lane; j < sc.count; j += 64) sum += sc.partials[(size_t)m * sc.count + j];
-      sum = wave_sum(sum);
-      if (lane == 0) row_factor[m] = 1.0f / sqrtf(sum * sc.inv_n + sc.eps);
-    }
-  }
   // workgroup b takes tile (b % tiles_per_group) of group (b / tiles_per_group): rows
   // r1 .. r1+15 and r1 + pair_offset .. of W. SiLU: one group, tiles over I. Rope: a
   // group is a head (group_rows = D), its tiles cover the first half of the head.
@@ -359,21 +350,49 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
 
   const int kb = wave * k_per_wave;
   const int ke = min(K, kb + k_per_wave);
-  for (int k = kb; k < ke; k += 32 * U) {
-    GsFrag w1[U], w2[U], xf[U];
+  GsFrag w1[U], w2[U], xf[U];
+  auto load_w = [&](int k) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int kk = k + 32 * u;
-      const bool ok = kk + 8 * lg < ke;
-      w1[u].u = (ok && wrow) ? *reinterpret_cast<const uint4*>(wp1 + kk) : make_uint4(0, 0, 0, 0);
-      w2[u].u = (ok && wrow) ? *reinterpret_cast<const uint4*>(wp2 + kk) : make_uint4(0, 0, 0, 0);
-      xf[u].u = (ok && ln < M) ? *reinterpret_cast<const uint4*>(xp + kk) : make_uint4(0, 0, 0, 0);
+      const bool ok = k + 32 * u + 8 * lg < ke && wrow;
+      w1[u].u = ok ? *reinterpret_cast<const uint4*>(wp1 + k + 32 * u) : make_uint4(0, 0, 0, 0);
+      w2[u].u = ok ? *reinterpret_cast<const uint4*>(wp2 + k + 32 * u) : make_uint4(0, 0, 0, 0);
     }
+  };
+  auto load_x = [&](int k) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bool ok = k + 32 * u + 8 * lg < ke && ln < M;
+      xf[u].u = ok ? *reinterpret_cast<const uint4*>(xp + k + 32 * u) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  // The first weights set out before anything else: they come from HBM and are what the
+  // kernel's time goes to. The rows' factors (a few dependent reads of L2) are worked out
+  // while they fly; x, which lies in L2, follows.
+  int k = kb;
+  if (k < ke) load_w(k);
+  if (sc.partials != nullptr) {
+    // the waves share the rows; a row's partial sums are added in a fixed order
+    for (int m = wave; m < M; m += nwaves) {
+      const float* row = sc.partials + (size_t)m * sc.count;
+      float sum = 0.f;
+      for (int j = lane; j < sc.count; j += 128) {
+        const float a = row[j], b = j + 64 < sc.count ? row[j + 64] : 0.f;
+        sum += a + b;
+      }
+      sum = wave_sum(sum);
+      if (lane == 0) row_factor[m] = 1.0f / sqrtf(sum * sc.inv_n + sc.eps);
+    }
+  }
+  while (k < ke) {
+    load_x(k);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, xf[u].v, acc1, 0, 0, 0);
       acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2[u].v, xf[u].v, acc2, 0, 0, 0);
     }
+    k += 32 * U;
+    if (k < ke) load_w(k);
   }
   if (nwaves > 1) {
     *reinterpret_cast<gs_f32x4_t*>(red + (((size_t)wave * 2 + 0) * 64 + lane) * 4) = acc1;
