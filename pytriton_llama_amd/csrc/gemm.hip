@@ -151,16 +151,24 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
 
   const int kb = wave * k_per_wave;
   const int ke = min(K, kb + k_per_wave);
-  for (int k = kb; k < ke; k += 32 * U) {
-    GsFrag wf[U], xf[MT][U];
+  // Two sets of weight registers: the loads of the next 32 U columns are under way while
+  // this set is multiplied, and a wave with at most 64 U columns has asked for all of its
+  // weights before it waits for any. x, which lies in L2, is fetched as it is needed.
+  GsFrag wa[U], wb[U], xf[MT][U];
+  auto load_w = [&](GsFrag (&wf)[U], int k) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int kk = k + 32 * u;
-      const bool ok = kk + 8 * lg < ke;
-      wf[u].u = (ok && wrow) ? *reinterpret_cast<const uint4*>(wp + kk) : make_uint4(0, 0, 0, 0);
+      const bool ok = k + 32 * u + 8 * lg < ke && wrow;
+      wf[u].u = ok ? *reinterpret_cast<const uint4*>(wp + k + 32 * u) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto multiply = [&](GsFrag (&wf)[U], int k) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bool ok = k + 32 * u + 8 * lg < ke;
 #pragma unroll
       for (int t = 0; t < MT; ++t)   // columns past the last row of x are never stored: no load
-        xf[t][u].u = (ok && 16 * t + ln < M) ? *reinterpret_cast<const uint4*>(xp[t] + kk)
+        xf[t][u].u = (ok && 16 * t + ln < M) ? *reinterpret_cast<const uint4*>(xp[t] + k + 32 * u)
                                              : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
@@ -168,6 +176,15 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
 #pragma unroll
       for (int t = 0; t < MT; ++t)
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u].v, xf[t][u].v, acc[t], 0, 0, 0);
+  };
+  if (kb < ke) load_w(wa, kb);
+  for (int k = kb; k < ke; k += 64 * U) {
+    const int k1 = k + 32 * U, k2 = k + 64 * U;
+    if (k1 < ke) load_w(wb, k1);
+    multiply(wa, k);
+    if (k1 >= ke) break;
+    if (k2 < ke) load_w(wa, k2);
+    multiply(wb, k1);
   }
 
   if (nwaves > 1) {
@@ -264,7 +281,7 @@ extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int M
     return PTL_ERR_ARG;
   if (M <= 16) return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
   if (M <= 32) return launch_skinny<2, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
-  return launch_skinny<4, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
+  return launch_skinny<4, 2>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
 }
 
 // How many partial sums a row gets from ptl_gemm_skinny_add_norm_bf16 with N columns.
@@ -369,6 +386,15 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   // The first weights set out before anything else: they come from HBM and are what the
   // kernel's time goes to. The rows' factors (a few dependent reads of L2) are worked out
   // while they fly; x, which lies in L2, follows.
+  // The loads are answered in the order they were asked: the partial sums of this wave's row
+  // first (a wait for them then leaves the weights under way), then the first weights, which
+  // come from HBM and are what the kernel's time goes to; the row's factor is worked out while
+  // they fly, and x, which lies in L2, follows.
+  const bool my_row = sc.partials != nullptr && wave < M;
+  const float* prow = sc.partials + (size_t)(my_row ? wave : 0) * sc.count;
+  float part[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) part[u] = (my_row && lane + 64 * u < sc.count) ? prow[lane + 64 * u] : 0.f;
   int k = kb;
   if (k < ke) load_w(k);
   if (sc.partials != nullptr) {
@@ -376,9 +402,11 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     for (int m = wave; m < M; m += nwaves) {
       const float* row = sc.partials + (size_t)m * sc.count;
       float sum = 0.f;
-      for (int j = lane; j < sc.count; j += 128) {
-        const float a = row[j], b = j + 64 < sc.count ? row[j + 64] : 0.f;
-        sum += a + b;
+      if (m == wave) {
+        sum = (part[0] + part[1]) + (part[2] + part[3]);
+        for (int j = lane + 256; j < sc.count; j += 64) sum += row[j];
+      } else {
+        for (int j = lane; j < sc.count; j += 64) sum += row[j];
       }
       sum = wave_sum(sum);
       if (lane == 0) row_factor[m] = 1.0f / sqrtf(sum * sc.inv_n + sc.eps);
