@@ -375,10 +375,19 @@ attn_decode_merge_kernel(T* __restrict__ out, long out_stride, const int32_t* __
                          const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                          int Hq, int D, int num_splits) {
   // one wave per (sequence, head): lanes take the splits' (max, denominator) side by side,
-  // then the head dimension, with the splits' weights in LDS
+  // then the head dimension, with the splits' weights in LDS. The partial results come from
+  // other compute units' writes, a long way off: the first 16 splits of the lane's first
+  // column are asked for before anything is computed, so that one wait covers them and the
+  // (max, denominator) pairs.
+  constexpr int AHEAD = 16;
   __shared__ float wgt[1024];
   const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const size_t base = ((size_t)seq * Hq + head) * num_splits;
+  const float* pa0 = part_acc + base * D + lane;
+  float first[AHEAD];
+#pragma unroll
+  for (int s = 0; s < AHEAD; ++s) first[s] = (s < num_splits && lane < D) ? pa0[(size_t)s * D] : 0.f;
+  const int row = q_start[seq];
   float mn = -INFINITY;
   for (int s = lane; s < num_splits; s += 64) mn = fmaxf(mn, part_ml[(base + s) * 2]);
   mn = wave_max(mn);
@@ -392,12 +401,17 @@ attn_decode_merge_kernel(T* __restrict__ out, long out_stride, const int32_t* __
   ll = wave_sum(ll);
   __syncthreads();
   const float inv = ll > 0.f ? 1.0f / ll : 0.f;
-  const int row = q_start[seq];
   for (int d = lane; d < D; d += 64) {
     float a = 0.f;
     const float* pa = part_acc + base * D + d;
+    int s = 0;
+    if (d == lane) {
+#pragma unroll
+      for (; s < AHEAD; ++s)
+        if (s < num_splits) a = fmaf(first[s], wgt[s], a);
+    }
 #pragma unroll 8
-    for (int s = 0; s < num_splits; ++s) a = fmaf(pa[(size_t)s * D], wgt[s], a);
+    for (; s < num_splits; ++s) a = fmaf(pa[(size_t)s * D], wgt[s], a);
     out[(size_t)row * out_stride + (size_t)head * D + d] = from_float<T>(a * inv);
   }
 }
