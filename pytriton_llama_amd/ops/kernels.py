@@ -556,10 +556,16 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
+SAMPLE_WIDE_FROM = 16384      # rows at least this long are sampled by many workgroups a row
+SAMPLE_WIDE_UP_TO = 64 * 4096
+
+
 def sample_top_p(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
-                 uniform: torch.Tensor, return_probs: bool = False):
+                 uniform: torch.Tensor, return_probs: bool = False, wide: Optional[bool] = None):
     """One token per row from the nucleus of softmax(logits / temperature).
-    temperature, top_p, uniform: float32 [R] on the GPU."""
+    temperature, top_p, uniform: float32 [R] on the GPU. ``wide``: spread a row over
+    many workgroups (several kernels; None: for rows of vocabulary size) or keep it
+    in one (one kernel); both follow the same rule."""
     _need_gpu(logits, temperature, top_p, uniform)
     if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelError("sample_top_p: logits must be float32 [R, V] with dense rows")
@@ -567,12 +573,25 @@ def sample_top_p(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.T
     for name, t in (("temperature", temperature), ("top_p", top_p), ("uniform", uniform)):
         if t.dtype != torch.float32 or t.numel() != R or not t.is_contiguous():
             raise KernelError(f"sample_top_p: {name} must be float32 [{R}]")
+    if wide is None:
+        wide = SAMPLE_WIDE_FROM <= V <= SAMPLE_WIDE_UP_TO
+    elif wide and V > SAMPLE_WIDE_UP_TO:
+        raise KernelError(f"sample_top_p: the many-workgroup form takes rows up to {SAMPLE_WIDE_UP_TO}")
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     probs = torch.empty((R, V), dtype=torch.float32, device=logits.device)   # scratch, then result
     lib = library.load("sampling")
-    _check(lib.ptl_sample_top_p(_ptr(out), _ptr(probs), int(return_probs), _ptr(logits), R, V,
-                                ctypes.c_long(logits.stride(0)), _ptr(temperature), _ptr(top_p),
-                                _ptr(uniform), _stream()), "sample_top_p")
+    if wide:
+        lib.ptl_sample_top_p_wide_workspace.restype = ctypes.c_size_t
+        nbytes = int(lib.ptl_sample_top_p_wide_workspace(R, V))
+        ws = torch.empty((nbytes // 4,), dtype=torch.float32, device=logits.device)
+        _check(lib.ptl_sample_top_p_wide(_ptr(out), _ptr(probs), int(return_probs), _ptr(logits), R, V,
+                                         ctypes.c_long(logits.stride(0)), _ptr(temperature),
+                                         _ptr(top_p), _ptr(uniform), _ptr(ws), _stream()),
+               "sample_top_p")
+    else:
+        _check(lib.ptl_sample_top_p(_ptr(out), _ptr(probs), int(return_probs), _ptr(logits), R, V,
+                                    ctypes.c_long(logits.stride(0)), _ptr(temperature), _ptr(top_p),
+                                    _ptr(uniform), _stream()), "sample_top_p")
     return (out, probs) if return_probs else out
 
 

@@ -562,6 +562,42 @@ def test_sample_top_p_frequencies(ops):
     assert freq[want == 0].sum() == 0
 
 
+@pytest.mark.parametrize("V", [16384, 20000, 128256])
+def test_sample_top_p_one_and_many_workgroups_a_row_agree(ops, V):
+    """The one-kernel and the many-workgroup samplers follow the same rule: the same nucleus
+    (up to a token at its edge, where float32 sums taken in another order meet top_p) and the
+    same draw, for peaked, ordinary and flat rows, top_p from almost 0 to 1, -inf and NaN
+    logits, and u at both ends."""
+    g = torch.Generator().manual_seed(V)
+    R = 12
+    logits = torch.randn(R, V, generator=g)
+    scale = torch.tensor([8.0, 4.0, 2.0, 1.0, 0.3, 0.02, 3.0, 3.0, 3.0, 3.0, 3.0, 1e-3]).view(R, 1)
+    logits = logits * scale
+    logits[6, ::3] = float("-inf")
+    logits[7, 5] = float("nan")
+    logits[8, V - 1] = 30.0                                  # the last token holds the mass
+    t = torch.tensor([0.6, 1.0, 0.8, 1.5, 1.0, 1.0, 0.7, 0.7, 0.7, 0.7, 0.7, 1.0])
+    p = torch.tensor([0.9, 0.9, 0.5, 0.95, 0.9, 0.9, 0.9, 0.9, 0.9, 1.0, 1e-6, 0.37])
+    u = torch.tensor([0.0, 0.3, 0.999999, 0.5, 0.77, 0.123, 0.9, 0.2, 0.5, 0.6, 0.4, 0.999])
+    args = [a.cuda() for a in (logits, t, p, u)]
+    tok1, pr1 = ops.sample_top_p(*args, return_probs=True, wide=False)
+    tokw, prw = ops.sample_top_p(*args, return_probs=True, wide=True)
+    tokw2 = ops.sample_top_p(*args, wide=True)
+    assert tokw.tolist() == tokw2.tolist()                    # the same call, the same tokens
+    for r in range(R):
+        a, b = pr1[r].double().cpu(), prw[r].double().cpu()
+        assert abs(float(b.sum()) - 1) < 1e-4
+        assert float((a - b).abs().sum()) < 2e-3, r
+        # the draw: same token, or a neighbour in the cumulative distribution
+        ca = torch.cumsum(b, 0)
+        assert int(tokw[r]) == int(tok1[r]) or abs(float(ca[int(tokw[r])] - ca[int(tok1[r])])) < 1e-3, r
+        assert b[int(tokw[r])] > 0
+    assert int(tokw[8]) == V - 1 and int(tokw[10]) == int(torch.argmax(logits[10]))
+    for r in (0, 2, 4):                                       # against the plain rule
+        want = plain_llama.top_p_probs(torch.nan_to_num(logits[r], nan=float("-inf")), float(t[r]), float(p[r]))
+        assert float((prw[r].double().cpu() - want).abs().sum()) < 1e-3
+
+
 def test_kernels_refuse_cpu_tensors(ops):
     with pytest.raises(ops.KernelError):
         ops.silu_mul(torch.zeros(2, 4))
