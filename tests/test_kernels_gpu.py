@@ -83,7 +83,10 @@ def test_gemm_nt(ops, dtype, mnk):
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["to_bf16", "to_fp32"])
 @pytest.mark.parametrize("mnk", [(1, 300, 72), (7, 65, 136), (16, 3072, 2048), (17, 100, 200),
-                                 (33, 16, 8192), (64, 1000, 64), (8, 2048, 8192), (5, 130, 2056)])
+                                 (33, 16, 8192), (64, 1000, 64), (8, 2048, 8192), (5, 130, 2056),
+                                 # a W wide enough for the streaming form: tiles past the end, K with a
+                                 # partial last batch, one row and sixteen
+                                 (1, 16384, 256), (8, 20003, 328), (16, 17000, 2048), (3, 40001, 72)])
 def test_gemm_skinny(ops, out_dtype, mnk):
     M, N, K = mnk
     torch.manual_seed(7)
