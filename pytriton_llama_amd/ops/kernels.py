@@ -41,7 +41,9 @@ def _ptr(t: Optional[torch.Tensor]):
 
 
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # torch's current stream as a raw handle (the two calls below take a fraction of a
+    # microsecond; torch.cuda.current_stream() builds a Stream object and takes ten)
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
 
 
 def _check(code: int, what: str) -> None:
@@ -208,6 +210,36 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     _check(lib.ptl_gemm_skinny_bf16(_ptr(y), _ptr(x), _ptr(w), M, N, K, ctypes.c_long(ldx),
                                     ctypes.c_long(N), _F32 if out_dtype == torch.float32 else _BF16,
                                     _stream()), "gemm_skinny")
+    return y
+
+
+def gemm_library_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``gemm_library`` takes x [M, K] and w [N, K]: bfloat16, dense rows of w,
+    16-byte aligned rows of both."""
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 2
+            and x.shape[1] == w.shape[1] and x.stride(1) == 1 and w.is_contiguous()
+            and x.shape[1] % 8 == 0 and (x.shape[0] == 1 or x.stride(0) % 8 == 0)
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_library(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y = x @ w.T by hipBLASLt, called directly with the descriptors and the algorithm of
+    the shape kept from its first call (see csrc/blaslt.hip). Output bfloat16 or float32."""
+    _need_gpu(x, w)
+    if not gemm_library_fits(x, w):
+        raise KernelError("gemm_library: needs bfloat16 x [M, K] and w [N, K] with K a multiple of 8 "
+                          "and 16-byte aligned rows")
+    M, K = x.shape
+    N = w.shape[0]
+    out_dtype = out_dtype or torch.bfloat16
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError("gemm_library: output is bfloat16 or float32")
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    ldx = x.stride(0) if M > 1 else max(K, 8)
+    lib = library.load("blaslt")
+    _check(lib.ptl_blaslt_gemm_bf16(_ptr(y), _ptr(x), _ptr(w), M, N, K, ctypes.c_long(ldx),
+                                    ctypes.c_long(N), _F32 if out_dtype == torch.float32 else _BF16,
+                                    _stream()), "gemm_library")
     return y
 
 

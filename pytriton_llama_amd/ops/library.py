@@ -26,10 +26,12 @@ HIPCC_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-shared", "-std=c++17"
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 KERNEL_LIBRARIES = ("embedding", "norm", "rope", "attention", "attention_prefill", "activation",
-                    "gemm", "sampling", "probe")
+                    "gemm", "blaslt", "sampling", "probe")
 # options of single sources. attention_prefill: no value there is a NaN unless an input is, and
 # without the promise every maximum of scores is preceded by instructions that quiet its inputs
 EXTRA_FLAGS = {"attention_prefill": ["-fno-honor-nans"]}
+# libraries a source is linked with (after the source on the command line)
+LINK_FLAGS = {"blaslt": ["-lhipblaslt"]}
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -94,7 +96,7 @@ def is_stale(name: str) -> bool:
 
 def compile_command(name: str, out: str) -> List[str]:
     return ([_hipcc()] + HIPCC_FLAGS + EXTRA_FLAGS.get(name, []) +
-            ["-I", CSRC_DIR, "-o", out, source_path(name)])
+            ["-I", CSRC_DIR, "-o", out, source_path(name)] + LINK_FLAGS.get(name, []))
 
 
 def build(names: Iterable[str] = KERNEL_LIBRARIES, force: bool = False, verbose: bool = True) -> None:

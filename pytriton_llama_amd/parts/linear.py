@@ -5,7 +5,8 @@ lite_llama/models/llama.py:37-40,61,120,221). Here: float32 always goes through
 the package's own vector-FMA kernel (a true 32-bit product, no reduced-precision
 matrix mode can be switched on underneath it); bfloat16 uses the package's
 skinny weight-streaming kernel for the few rows of a decode step and the
-library product (hipBLASLt through torch) for the many rows of a prompt.
+library product (hipBLASLt, called directly: ops.gemm_library) for the many rows
+of a prompt.
 """
 from __future__ import annotations
 
@@ -15,7 +16,7 @@ import torch
 
 from .. import ops
 
-LINEAR_LIBRARIES = ("gemm",)
+LINEAR_LIBRARIES = ("gemm", "blaslt")
 SKINNY_ROWS = 8          # rows up to which the skinny kernel takes a bfloat16 product
 SKINNY_ROWS_F32 = 16     # ... when float32 output is wanted (the head)
 
@@ -32,8 +33,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     # library up to 8 rows (and ahead for the vocabulary-sized head); beyond that the library
     if ops.gemm_skinny_fits(x, w) and (M <= SKINNY_ROWS or (to_f32 and M <= SKINNY_ROWS_F32)):
         return ops.gemm_skinny(x, w, out_dtype)
+    if ops.gemm_library_fits(x, w):
+        return ops.gemm_library(x, w, out_dtype)
     if to_f32:
-        if x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
-            return torch.mm(x, w.t(), out_dtype=torch.float32)
         return ops.gemm_nt(x, w, torch.float32)
-    return torch.nn.functional.linear(x, w)
+    return torch.nn.functional.linear(x, w)         # (rows that are not 16-byte aligned)

@@ -108,6 +108,32 @@ def test_gemm_skinny(ops, out_dtype, mnk):
         ops.gemm_skinny(x[:, :K - 4], w[:, :K - 4].contiguous())
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["to_bf16", "to_fp32"])
+@pytest.mark.parametrize("mnk", [(1, 300, 72), (17, 100, 200), (64, 3072, 2048), (300, 130, 136),
+                                 (512, 2048, 2048), (777, 1000, 328), (2048, 352, 176)])
+def test_gemm_library(ops, out_dtype, mnk):
+    """The library product called directly: against a float64 product, also for rows of x that
+    are a slice of a wider buffer, twice (the second call takes the kept plan)."""
+    M, N, K = mnk
+    torch.manual_seed(9)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    want = (x.double() @ w.double().T).float()
+    t = dict(atol=1e-4, rtol=1e-4) if out_dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    for _ in range(2):
+        y = ops.gemm_library(x, w, out_dtype)
+        assert y.dtype == out_dtype and y.shape == (M, N)
+        torch.testing.assert_close(y.float(), want, **t)
+    wide = torch.randn(M, K + 24, device="cuda").to(torch.bfloat16)
+    xs = wide[:, 8:8 + K]
+    torch.testing.assert_close(ops.gemm_library(xs, w, out_dtype).float(),
+                               (xs.double() @ w.double().T).float(), **t)
+    assert not ops.gemm_library_fits(wide[:, 1:1 + K], w)            # rows not 16-byte aligned
+    assert not ops.gemm_library_fits(x.float(), w)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_library(x.float(), w)
+
+
 @pytest.mark.parametrize("mik", [(1, 176, 64), (8, 8192, 2048), (16, 320, 136), (5, 48, 2056)])
 def test_gate_up_silu(ops, mik):
     M, I, K = mik
