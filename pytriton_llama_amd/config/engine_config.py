@@ -41,7 +41,8 @@ class EngineConfig:
     prefill_chunk: Optional[int] = None      # largest portion of one prompt in a step
     max_model_len: int = 2048                # reference: max_seq_len
     seed: int = 0
-    use_graphs: bool = True                  # replay decode-only steps as HIP graphs
+    use_graphs: bool = True                  # replay decode-only steps, and steps that bring one
+                                             # portion of one prompt (up to 1,024 tokens), as HIP graphs
     async_decode: bool = True                # launch a decode step before the tokens of the one
                                              # before it have reached the host
 

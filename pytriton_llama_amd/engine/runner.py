@@ -32,9 +32,12 @@ class ModelRunner:
         self.storage = CacheStorage(self.manager, model.dtype, self.device)
         # decode-only steps replay a HIP graph when the longest request is known
         self.graphs = None
+        self.portion_graphs = None
         if use_graphs and max_model_len and self.device.type == "cuda" and not self.manager.states:
-            from .graphs import DecodeGraphs
+            from .graphs import DecodeGraphs, PortionGraphs
             self.graphs = DecodeGraphs(model, self.manager, self.storage, max_model_len, self.device)
+            self.portion_graphs = PortionGraphs(model, self.manager, self.storage, max_model_len,
+                                                self.device)
 
     def admit(self, request: Hashable) -> None:
         slot = self.manager.admit(request)
@@ -57,6 +60,8 @@ class ModelRunner:
             logits = self.graphs.step(entries, token_feed)
         elif token_feed is not None:
             raise ValueError("only steps that replay a graph can take their tokens from the device")
+        elif self.portion_graphs is not None and self.portion_graphs.fits(entries):
+            logits = self.portion_graphs.step(entries)
         else:
             ctx, _ = build_context(entries, self.manager, self.device, self.model.vocab_size)
             logits = self.model.forward(ctx, self.storage)

@@ -170,6 +170,67 @@ def test_decode_graphs_match_eager_steps(folder_b, dtype):
     assert replays == 40
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_portion_graphs_match_eager_steps(folder_a, folder_b, which, dtype):
+    """Steps that bring one portion of one prompt, replayed as HIP graphs (padded to 32, 64,
+    ... tokens), give the logits of the same steps launched kernel by kernel: every replay is
+    checked, with a prefix already in the cache, the wanted place last, in the middle or
+    absent, steps of other kinds and a request's end between the replays, and pages that are
+    used again."""
+    from pytriton_llama_amd.config import build_model, read_config_json
+    from pytriton_llama_amd.engine.batch import StepEntry
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_weights
+    folder, page = folder_a if which == "A" else folder_b
+    cfg = read_config_json(folder)
+    model = build_model(cfg)
+    load_weights(model, folder, dtype, "cuda:0")
+    pages = -(-520 // page)                                # not many more than are held at once
+    eager = ModelRunner(model, page, pages, 4)
+    graphed = ModelRunner(model, page, pages, 4, max_model_len=260, use_graphs=True)
+    assert graphed.portion_graphs is not None and eager.portion_graphs is None
+    g = torch.Generator().manual_seed(13)
+    toks = {r: torch.randint(0, model.vocab_size, (260,), generator=g).tolist() for r in "abc"}
+    fed = {r: 0 for r in toks}
+    # float32: the same arithmetic on both sides. bfloat16: a padded portion takes the library
+    # products where the eager step of up to 16 rows takes the fused kernels, so the two differ
+    # as two bfloat16 runs do (the tolerance of the engine against the plain implementation).
+    tol = 1e-5 if dtype == torch.float32 else 4e-2
+
+    def both(spec):
+        entries = []
+        for r, n, want in spec:
+            entries.append(StepEntry(r, toks[r][fed[r]:fed[r] + n], want))
+            fed[r] += n
+        le = eager.step(entries).float().cpu()
+        lg = graphed.step(entries).float().cpu()
+        assert le.shape == lg.shape
+        if le.numel():
+            assert float((le - lg).abs().max()) / float(le.abs().max()) < tol
+
+    both([("a", 2, [1])])                                   # bucket of 32
+    both([("a", 31, [30])])
+    both([("a", 33, [7])])                                  # bucket of 64, a place in the middle
+    both([("b", 70, [])])                                   # bucket of 128, nothing wanted
+    both([("b", 5, [4]), ("a", 1, [0])])                    # a mixed step: eager in both
+    both([("a", 64, [63])])
+    for i in range(12):                                     # the same buckets again and again
+        both([("a" if i % 2 else "b", 3 + i, [2 + i])])
+        if i == 5:
+            both([("b", 1, [0])])                           # a decode step (its own graph)
+            torch.cuda.synchronize()
+    for r in (eager, graphed):
+        r.end("a")
+    toks["a"] = toks["a"][::-1]
+    fed["a"] = 0
+    both([("a", 100, [99])])                                # a new request in the freed pages
+    both([("c", 40, [39])])
+    both([("c", 129, [128])])                               # bucket of 256
+    used = graphed.portion_graphs.buckets
+    assert sorted(used) == [32, 64, 128, 256] and all(b.graph is not None for b in used.values())
+
+
 def test_logprobs_of_generated_tokens(folder_a):
     """log_softmax of the plain logits at the tokens the engine chose."""
     from pytriton_llama_amd.generate import GenerateText
