@@ -222,11 +222,13 @@ def gemm_library_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def gemm_library(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def gemm_library(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                 checked: bool = False) -> torch.Tensor:
     """y = x @ w.T by hipBLASLt, called directly with the descriptors and the algorithm of
-    the shape kept from its first call (see csrc/blaslt.hip). Output bfloat16 or float32."""
+    the shape kept from its first call (see csrc/blaslt.hip). Output bfloat16 or float32.
+    ``checked``: the caller has just asked ``gemm_library_fits``."""
     _need_gpu(x, w)
-    if not gemm_library_fits(x, w):
+    if not checked and not gemm_library_fits(x, w):
         raise KernelError("gemm_library: needs bfloat16 x [M, K] and w [N, K] with K a multiple of 8 "
                           "and 16-byte aligned rows")
     M, K = x.shape

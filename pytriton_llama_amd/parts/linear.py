@@ -31,10 +31,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     to_f32 = out_dtype == torch.float32
     # measured on MI355X at the 1B shapes: the weight-streaming kernel is level with the
     # library up to 8 rows (and ahead for the vocabulary-sized head); beyond that the library
-    if ops.gemm_skinny_fits(x, w) and (M <= SKINNY_ROWS or (to_f32 and M <= SKINNY_ROWS_F32)):
+    if (M <= SKINNY_ROWS or (to_f32 and M <= SKINNY_ROWS_F32)) and ops.gemm_skinny_fits(x, w):
         return ops.gemm_skinny(x, w, out_dtype)
     if ops.gemm_library_fits(x, w):
-        return ops.gemm_library(x, w, out_dtype)
+        return ops.gemm_library(x, w, out_dtype, checked=True)
     if to_f32:
         return ops.gemm_nt(x, w, torch.float32)
     return torch.nn.functional.linear(x, w)         # (rows that are not 16-byte aligned)
