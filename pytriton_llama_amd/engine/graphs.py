@@ -11,10 +11,11 @@ graph is replayed. Rows beyond the live sequences are padding: they have
 ctx_len 0 (attention reads nothing), slot -1 (nothing is written to the cache)
 and their logits are dropped.
 
-A step with a single entry of several tokens (a prompt, or a portion of one, alone in the
-step: the first thing a request sees on an idle engine) is some 150 launches that cost the
+A step with one entry of several tokens (a prompt, or a portion of one: the first thing a
+request sees on an engine that is idle or only decoding) is some 150 launches that cost the
 host about 2.4 ms at 16 layers, more than the GPU needs for up to a thousand tokens. Such a
-step runs through a graph captured once per bucket of its token count (32, 64, ... 1024):
+step runs through a graph captured once per bucket of its token count (32, 64, ... 1024) and
+of the number of single-token entries beside it (0, 1, 2, 4, ...):
 the tokens are padded to the bucket with rows that write nothing to the cache (slot -1) and
 that no query block covers (the work lists name blocks up to the bucket's size; a block
 past the real tokens is empty and its workgroup leaves at once).
@@ -194,24 +195,26 @@ class DecodeGraphs:
 
 
 PORTION_BUCKETS = (32, 64, 128, 256, 512, 1024)
+MAX_PORTION_GRAPHS = 32          # pairs of (decoding rows, portion size) kept; others run eagerly
 
 
 class _PortionBucket:
-    """Static buffers, context and captured graph for one padded token count of a
-    single-entry step."""
+    """Static buffers, context and captured graph for a step of ``rows`` single-token entries
+    (padded) followed by one entry of up to ``size`` tokens (padded)."""
 
-    def __init__(self, size: int, manager, width: int, max_model_len: int, device):
+    def __init__(self, rows: int, size: int, manager, width: int, max_model_len: int, device):
         from .batch import GENERIC_BLOCK_ROWS, MFMA_BIG_BLOCK_ROWS, MFMA_BLOCK_ROWS
-        self.size = T = size
+        self.rows, self.size = B, T = rows, size
         G = len(manager.paged)
         blocks = {"16": GENERIC_BLOCK_ROWS, "64": MFMA_BLOCK_ROWS, "128": MFMA_BIG_BLOCK_ROWS}
-        names = [("token_ids", T), ("positions", T), ("ctx_len", 1), ("state_slots", 1),
-                 ("q_start", 2), ("logit_rows", 1)]
-        for tag, rows in blocks.items():
-            n = -(-T // rows)
+        names = [("token_ids", B + T), ("positions", B + T), ("ctx_len", B + 1),
+                 ("state_slots", B + 1), ("q_start", B + 2), ("logit_rows", B + 1)]
+        for tag, r in blocks.items():
+            n = -(-T // r)
             names += [("ws_" + tag, n), ("wo_" + tag, n)]
+        names += [("ws_all16", B + -(-T // GENERIC_BLOCK_ROWS)), ("wo_all16", B + -(-T // GENERIC_BLOCK_ROWS))]
         for g in range(G):
-            names += [(f"slots{g}", T), (f"table{g}", width)]
+            names += [(f"slots{g}", B + T), (f"table{g}", (B + 1) * width)]
         self.spans, n = {}, 0
         for name, k in names:
             self.spans[name] = (n, k)
@@ -219,21 +222,33 @@ class _PortionBucket:
         self.host = torch.zeros(n, dtype=torch.int32).pin_memory()
         self.np = self.host.numpy()
         self.dev = torch.zeros(n, dtype=torch.int32, device=device)
-        for tag, rows in blocks.items():               # blocks of the one sequence, last rows first
-            self.view_np("wo_" + tag)[:] = np.arange(0, T, rows)[::-1]
+        # the portion is sequence B of the step; its query blocks, last rows first
+        for tag, r in blocks.items():
+            self.view_np("ws_" + tag)[:] = B
+            self.view_np("wo_" + tag)[:] = np.arange(0, T, r)[::-1]
+        # every sequence in 16-row blocks (the kernel that takes the other head sizes)
+        n16 = -(-T // GENERIC_BLOCK_ROWS)
+        self.view_np("ws_all16")[:n16] = B
+        self.view_np("wo_all16")[:n16] = np.arange(0, T, GENERIC_BLOCK_ROWS)[::-1]
+        self.view_np("ws_all16")[n16:] = np.arange(B)
+        self.view_np("wo_all16")[n16:] = 0
+        self.view_np("q_start")[:B + 1] = np.arange(B + 1)
+        self.view_np("logit_rows")[:B] = np.arange(B)
         work = {tag: (self.view("ws_" + tag), self.view("wo_" + tag)) for tag in blocks}
-        groups = [GroupContext(self.view(f"table{g}").view(1, width), self.view(f"slots{g}"))
+        work["all16"] = (self.view("ws_all16"), self.view("wo_all16"))
+        groups = [GroupContext(self.view(f"table{g}").view(B + 1, width), self.view(f"slots{g}"))
                   for g in range(G)]
+        self.table_np = [self.view_np(f"table{g}").reshape(B + 1, width) for g in range(G)]
         self.ctx = StepContext(
             token_ids=self.view("token_ids"), positions=self.view("positions"),
             q_start=self.view("q_start"), ctx_len=self.view("ctx_len"),
             state_slots=self.view("state_slots"), logit_rows=self.view("logit_rows"),
-            work={"all16": work["16"], "multi16": work["16"], "multi64": work["64"],
+            work={"all16": work["all16"], "multi16": work["16"], "multi64": work["64"],
                   "multi128": work["128"]},
             groups=groups,
-            num_tokens=T, num_seqs=1, num_logit_rows=1, logit_rows_are_identity=False,
-            num_decode_seqs=0, q_lens=[T], ctx_lens=[max_model_len], max_q_len=T,
-            max_ctx_len=max_model_len)
+            num_tokens=B + T, num_seqs=B + 1, num_logit_rows=B + 1, logit_rows_are_identity=False,
+            num_decode_seqs=B, q_lens=[1] * B + [T], ctx_lens=[max_model_len] * (B + 1),
+            max_q_len=T, max_ctx_len=max_model_len)
         self.graph = None
         self.logits = None
         self.copied = None                 # event: the last copy of ``host`` has been made
@@ -248,7 +263,8 @@ class _PortionBucket:
 
 
 class PortionGraphs:
-    """Steps of a single entry with 2 to 1,024 tokens (and at most one wanted place)."""
+    """Steps of single-token entries (any number up to the largest decode bucket, also none)
+    and exactly one entry of 2 to 1,024 tokens with at most one wanted place."""
 
     def __init__(self, model, manager, storage, max_model_len: int, device):
         if manager.states:
@@ -258,50 +274,93 @@ class PortionGraphs:
         self.device = device
         self.max_model_len = int(max_model_len)
         self.width = -(-self.max_model_len // manager.page_size)
-        self.sizes = [s for s in PORTION_BUCKETS]
-        self.buckets: Dict[int, _PortionBucket] = {}
+        self.sizes = list(PORTION_BUCKETS)
+        self.row_sizes = [0] + bucket_sizes(manager.max_num_seqs)
+        self.buckets: Dict[tuple, _PortionBucket] = {}
+
+    def _split(self, entries):
+        """(indices of the single-token entries, index of the portion) or None."""
+        ones, portion = [], None
+        for i, e in enumerate(entries):
+            if len(e.tokens) == 1:
+                ones.append(i)
+            elif portion is None:
+                portion = i
+            else:
+                return None
+        return None if portion is None else (ones, portion)
 
     def fits(self, entries: Sequence[StepEntry]) -> bool:
-        if len(entries) != 1:
+        split = self._split(entries)
+        if split is None:
             return False
-        e = entries[0]
-        n = len(e.tokens)
-        return (2 <= n <= self.sizes[-1] and len(e.want) <= 1
-                and self.manager.num_tokens.get(e.request, 0) + n <= self.max_model_len)
+        ones, portion = split
+        if len(ones) > self.row_sizes[-1]:
+            return False
+        e = entries[portion]
+        if not (2 <= len(e.tokens) <= self.sizes[-1] and len(e.want) <= 1):
+            return False
+        for i in ones:
+            if list(entries[i].want) not in ([], [0]):
+                return False
+        key = (next(r for r in self.row_sizes if r >= len(ones)),
+               next(t for t in self.sizes if t >= len(e.tokens)))
+        if key not in self.buckets and len(self.buckets) >= MAX_PORTION_GRAPHS:
+            return False
+        return all(self.manager.num_tokens.get(x.request, 0) + len(x.tokens) <= self.max_model_len
+                   for x in entries)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Logits [wanted, vocab] (one row or none) of a step with one entry."""
+        """Logits [wanted, vocab] in the order of the entries."""
         m = self.manager
+        ones, portion = self._split(entries)
         tokens_of: list = []
-        start = take_pages(entries, m, self.model.vocab_size, tokens_of)[0]
-        e, toks = entries[0], tokens_of[0]
-        n = len(toks)
-        size = next(s for s in self.sizes if s >= n)
-        b = self.buckets.get(size)
+        starts = take_pages(entries, m, self.model.vocab_size, tokens_of)
+        e, toks, start = entries[portion], tokens_of[portion], starts[portion]
+        k, n = len(ones), len(toks)
+        key = (next(r for r in self.row_sizes if r >= k), next(t for t in self.sizes if t >= n))
+        b = self.buckets.get(key)
         if b is None:
-            b = self.buckets[size] = _PortionBucket(size, m, self.width, self.max_model_len,
-                                                    self.device)
-        # Portions without a wanted place are not waited for, so the host can be steps ahead of
-        # the GPU: the pinned buffer is written again only when its last copy has been made.
+            b = self.buckets[key] = _PortionBucket(key[0], key[1], m, self.width,
+                                                   self.max_model_len, self.device)
+        B = b.rows
+        # Steps that nobody waits for (nothing wanted) let the host run ahead of the GPU: the
+        # pinned buffer is written again only when its last copy has been made.
         if b.copied is not None:
             b.copied.synchronize()
         np_ = b.view_np
-        np_("token_ids")[:n] = toks
-        np_("token_ids")[n:] = 0
-        np_("positions")[:n] = np.arange(start, start + n)
-        np_("positions")[n:] = 0
-        np_("q_start")[:] = (0, n)
-        np_("ctx_len")[0] = start + n
-        np_("state_slots")[0] = m.slot_of[e.request]
-        np_("logit_rows")[0] = e.want[0] if e.want else n - 1
+        tok, pos, ctx = np_("token_ids"), np_("positions"), np_("ctx_len")
+        tok[:k] = [entries[i].tokens[0] for i in ones]
+        pos[:k] = [starts[i] for i in ones]
+        tok[k:B] = 0
+        pos[k:B] = 0
+        ctx[:k] = pos[:k] + 1
+        ctx[k:B] = 0                                     # padding rows: attention reads nothing
+        tok[B:B + n] = toks
+        tok[B + n:] = 0
+        pos[B:B + n] = np.arange(start, start + n)
+        pos[B + n:] = 0
+        ctx[B] = start + n
+        np_("q_start")[B + 1] = B + n
+        slot_of = np_("state_slots")
+        slot_of[:k] = [m.slot_of[entries[i].request] for i in ones]
+        slot_of[k:B] = 0
+        slot_of[B] = m.slot_of[e.request]
+        np_("logit_rows")[B] = B + (e.want[0] if e.want else n - 1)
+        P = m.page_size
         for g, group in enumerate(m.paged):
-            slots = np_(f"slots{g}")
-            slots[:n] = m.slot_array(e.request, g, start, n)
-            slots[n:] = -1
+            slots, table_np = np_(f"slots{g}"), b.table_np[g]
+            for j, i in enumerate(ones):
+                table = group.tables[entries[i].request]
+                slots[j] = table[starts[i] // P] * P + starts[i] % P
+                table_np[j, :len(table)] = table
+                table_np[j, len(table):] = -1
+            slots[k:B] = -1
+            slots[B:B + n] = m.slot_array(e.request, g, start, n)
+            slots[B + n:] = -1
             table = group.tables[e.request]
-            row = np_(f"table{g}")
-            row[:len(table)] = table
-            row[len(table):] = -1
+            table_np[B, :len(table)] = table
+            table_np[B, len(table):] = -1
         b.dev.copy_(b.host, non_blocking=True)
         if b.graph is None:
             b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device)
@@ -309,5 +368,11 @@ class PortionGraphs:
             b.copied = torch.cuda.Event()
         b.copied.record()
         b.graph.replay()
-        # (the logits are the graph's own buffer: the next replay of this bucket overwrites them)
-        return b.logits.clone() if e.want else b.logits[:0]
+        # rows of the graph's logits in the caller's order of entries (a copy: the next replay
+        # of this bucket overwrites the graph's own buffer)
+        row_of = {i: j for j, i in enumerate(ones)}
+        row_of[portion] = B
+        rows = [row_of[i] for i, x in enumerate(entries) if len(x.want)]
+        if not rows:
+            return b.logits[:0]
+        return b.logits.index_select(0, torch.tensor(rows, dtype=torch.int32, device=b.logits.device))

@@ -173,11 +173,11 @@ def test_decode_graphs_match_eager_steps(folder_b, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("which", ["A", "B"])
 def test_portion_graphs_match_eager_steps(folder_a, folder_b, which, dtype):
-    """Steps that bring one portion of one prompt, replayed as HIP graphs (padded to 32, 64,
-    ... tokens), give the logits of the same steps launched kernel by kernel: every replay is
-    checked, with a prefix already in the cache, the wanted place last, in the middle or
-    absent, steps of other kinds and a request's end between the replays, and pages that are
-    used again."""
+    """Steps that bring one portion of one prompt, alone or beside decoding requests, replayed
+    as HIP graphs (padded to 32, 64, ... tokens and 1, 2, 4, ... decoding rows), give the
+    logits of the same steps launched kernel by kernel: every replay is checked, with a prefix
+    already in the cache, the wanted place last, in the middle or absent, steps of other kinds
+    and a request's end between the replays, and pages that are used again."""
     from pytriton_llama_amd.config import build_model, read_config_json
     from pytriton_llama_amd.engine.batch import StepEntry
     from pytriton_llama_amd.engine.runner import ModelRunner
@@ -186,7 +186,7 @@ def test_portion_graphs_match_eager_steps(folder_a, folder_b, which, dtype):
     cfg = read_config_json(folder)
     model = build_model(cfg)
     load_weights(model, folder, dtype, "cuda:0")
-    pages = -(-520 // page)                                # not many more than are held at once
+    pages = -(-600 // page)                                # not many more than are held at once
     eager = ModelRunner(model, page, pages, 4)
     graphed = ModelRunner(model, page, pages, 4, max_model_len=260, use_graphs=True)
     assert graphed.portion_graphs is not None and eager.portion_graphs is None
@@ -213,7 +213,7 @@ def test_portion_graphs_match_eager_steps(folder_a, folder_b, which, dtype):
     both([("a", 31, [30])])
     both([("a", 33, [7])])                                  # bucket of 64, a place in the middle
     both([("b", 70, [])])                                   # bucket of 128, nothing wanted
-    both([("b", 5, [4]), ("a", 1, [0])])                    # a mixed step: eager in both
+    both([("b", 5, [4]), ("a", 1, [0])])                    # a decoding row beside the portion
     both([("a", 64, [63])])
     for i in range(12):                                     # the same buckets again and again
         both([("a" if i % 2 else "b", 3 + i, [2 + i])])
@@ -227,8 +227,16 @@ def test_portion_graphs_match_eager_steps(folder_a, folder_b, which, dtype):
     both([("a", 100, [99])])                                # a new request in the freed pages
     both([("c", 40, [39])])
     both([("c", 129, [128])])                               # bucket of 256
+    # decoding rows beside a portion, in any order of the entries, wanted or not
+    both([("a", 1, [0]), ("c", 9, []), ("b", 1, [])])
+    both([("c", 35, [0]), ("b", 1, [0]), ("a", 1, [0])])
+    for i in range(4):
+        both([("b", 1, [0]), ("c", 2 + i, [1 + i]), ("a", 1, [0])])
+        both([("a", 1, [0]), ("b", 1, [0])])                # decode-only steps between them
+    both([("a", 7, [6]), ("b", 3, [2])])                    # two portions: launched kernel by kernel
     used = graphed.portion_graphs.buckets
-    assert sorted(used) == [32, 64, 128, 256] and all(b.graph is not None for b in used.values())
+    assert {(0, 32), (0, 64), (0, 128), (0, 256), (1, 32), (2, 32), (2, 64)} <= set(used)
+    assert all(b.graph is not None for b in used.values())
 
 
 def test_logprobs_of_generated_tokens(folder_a):
