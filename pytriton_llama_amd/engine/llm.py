@@ -177,6 +177,42 @@ class Engine:
             self._collect(self._inflight)
             self._inflight = None
 
+    def warm_up(self, decode_batches: Optional[Sequence[int]] = None,
+                portion_sizes: Optional[Sequence[int]] = None) -> None:
+        """Capture the HIP graphs before the first request needs them (a capture takes about
+        0.1 s): decode steps of the given batch sizes (default: every bucket) and steps with
+        one prompt portion of the given sizes alone (default: every bucket that the token
+        budget and ``max_model_len`` allow). Only on an idle engine; the requests it makes up
+        are gone when it returns."""
+        if self.has_work:
+            raise RuntimeError("warm_up needs an idle engine")
+        runner = self.runner
+        if runner.graphs is None:
+            return
+        from .batch import StepEntry
+        limit = min(self.config.max_num_batched_tokens, self.config.max_model_len)
+        if portion_sizes is None:
+            portion_sizes = [t for t in runner.portion_graphs.sizes if t <= limit]
+        if decode_batches is None:
+            decode_batches = runner.graphs.sizes
+        for t in portion_sizes:
+            if self.manager_fits(t, 1):
+                runner.step([StepEntry(("warm-up", t), [0] * t, [t - 1])])
+                runner.end(("warm-up", t))
+        for b in decode_batches:
+            if b <= self.config.max_num_seqs and self.manager_fits(1, b):
+                names = [("warm-up", b, i) for i in range(b)]
+                runner.step([StepEntry(n, [0], [0]) for n in names])
+                for n in names:
+                    runner.end(n)
+        torch.cuda.synchronize()
+
+    def manager_fits(self, tokens_each: int, requests: int) -> bool:
+        """Whether the free pages hold ``requests`` new requests of ``tokens_each`` tokens."""
+        m = self.runner.manager
+        pages = -(-tokens_each // m.page_size) * requests
+        return all(g.pool.num_free >= pages for g in m.paged)
+
     # ---- whole generations ----------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]],
                  params: Union[SamplingParams, Sequence[SamplingParams], None] = None) -> List[List[int]]:

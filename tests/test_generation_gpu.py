@@ -239,6 +239,32 @@ def test_portion_graphs_match_eager_steps(folder_a, folder_b, which, dtype):
     assert all(b.graph is not None for b in used.values())
 
 
+def test_warm_up_captures_the_graphs_and_changes_nothing(folder_b):
+    """Engine.warm_up makes the graphs of every bucket the limits allow and gives everything
+    back; generation afterwards is what it is without it."""
+    from pytriton_llama_amd.config import EngineConfig
+    from pytriton_llama_amd.engine import Engine, SamplingParams
+    folder, page = folder_b
+    g = torch.Generator().manual_seed(3)
+    prompts = [torch.randint(0, 384, (n,), generator=g).tolist() for n in (20, 45, 3)]
+    params = SamplingParams(temperature=0.0, max_new_tokens=6, ignore_eos=True)
+
+    def engine():
+        return Engine(folder, EngineConfig(dtype="float32", page_size=page, num_pages=24, max_num_seqs=4,
+                                           max_model_len=128, max_num_batched_tokens=100))
+    plain = engine().generate(prompts, params)
+    eng = engine()
+    free = [g.pool.num_free for g in eng.runner.manager.paged]
+    eng.warm_up()
+    assert [g.pool.num_free for g in eng.runner.manager.paged] == free and not eng.has_work
+    assert sorted(eng.runner.portion_graphs.buckets) == [(0, 32), (0, 64)]      # 128 > the budget of 100
+    assert sorted(eng.runner.graphs.buckets) == [1, 2, 4]
+    assert eng.generate(prompts, params) == plain
+    eng.add_request(prompts[0], params)
+    with pytest.raises(RuntimeError):
+        eng.warm_up()
+
+
 def test_logprobs_of_generated_tokens(folder_a):
     """log_softmax of the plain logits at the tokens the engine chose."""
     from pytriton_llama_amd.generate import GenerateText
