@@ -184,7 +184,12 @@ sample_top_p_kernel(int32_t* __restrict__ out, float* __restrict__ work, int wan
   const float mc = mx * c;
   float z = 0.f;
   // (a NaN logit counts as -inf: probability 0)
-  auto expo = [&](float x) { return x != x ? 0.f : __builtin_amdgcn_exp2f(fmaf(x, c, -mc)); };
+  float emax = 0.f;                          // the largest e (1 up to rounding)
+  auto expo = [&](float x) {
+    const float e = x != x ? 0.f : __builtin_amdgcn_exp2f(fmaf(x, c, -mc));
+    emax = fmaxf(emax, e);
+    return e;
+  };
   if (vec_in && vec_ex) {
     const int n4 = V >> 2;
     auto exp4 = [&](int i, float4 x) {
@@ -218,6 +223,7 @@ sample_top_p_kernel(int32_t* __restrict__ out, float* __restrict__ work, int wan
     }
   }
   z = block_sum(z, scratch);                 // (its barriers also publish ex[] to the block)
+  emax = block_max(emax, scratch);
   const float tp = top_p[r] * z;             // all masses below are in units of e
   float thr = -1.0f;                         // kept: e > thr
   if (top_p[r] < 1.0f) {
@@ -323,8 +329,8 @@ sample_top_p_kernel(int32_t* __restrict__ out, float* __restrict__ work, int wan
         __syncthreads();
       }
       thr = thr_s;
-      // the most likely token (e = 1 up to rounding) is always kept: nothing lies before it
-      if (thr >= 0.9999f) thr = 0.9999f;
+      // the most likely token is always kept: nothing lies before it
+      if (thr >= emax) thr = __uint_as_float(__float_as_uint(emax) - 1u);
     }
   }
 
@@ -470,7 +476,8 @@ __device__ __forceinline__ uint32_t sw_key(float x) {
   const uint32_t b = __float_as_uint(x);
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
-__device__ __forceinline__ float sw_clean(float x) { return x != x ? -INFINITY : x; }
+// a NaN logit counts as -inf; -0 and +0 are one value (their bit patterns differ)
+__device__ __forceinline__ float sw_clean(float x) { return x != x ? -INFINITY : (x == 0.f ? 0.f : x); }
 
 struct SwScale {
   float mx, inv_w, c, mc, z;               // row max, buckets per unit of x, log2(e)/T, mx*c, sum of e

@@ -627,6 +627,34 @@ def test_sample_top_p_one_and_many_workgroups_a_row_agree(ops, V):
         assert float((prw[r].double().cpu() - want).abs().sum()) < 1e-3
 
 
+@pytest.mark.parametrize("wide", [False, True], ids=["one_workgroup", "many_workgroups"])
+def test_sample_top_p_nearly_flat_row_and_signed_zeros(ops, wide):
+    """A nearly flat row with a top_p that admits two tokens keeps exactly those two (the most
+    likely token is always kept, its neighbours only by the rule); +0 and -0 are one logit."""
+    V = 20000
+    g = torch.Generator().manual_seed(4)
+    flat = torch.randn(V, generator=g) * 1e-3
+    top = torch.topk(flat, 3).indices.tolist()
+    zeros = torch.zeros(V)
+    zeros[::2] = -0.0
+    zeros[[11, 500]] = torch.tensor([1.0, 0.5])
+    logits = torch.stack([flat, zeros]).cuda()
+    t = torch.ones(2).cuda()
+    # row 0: every token has about 1/V of the mass; the mass before the third token is ~2/V
+    # row 1: tokens 11 and 500 hold e + sqrt(e) of e + sqrt(e) + V - 2; 0.01 lets in the zeros' first
+    p = torch.tensor([1.5 / V, 0.01]).cuda()
+    u = torch.tensor([0.99, 0.5]).cuda()
+    tok, probs = ops.sample_top_p(logits, t, p, u, return_probs=True, wide=wide)
+    kept0 = torch.nonzero(probs[0]).flatten().tolist()
+    assert sorted(kept0) == sorted(top[:2]) and int(tok[0]) in kept0
+    want = plain_llama.top_p_probs(zeros, 1.0, 0.01)
+    got = probs[1].double().cpu()
+    # all zeros, whatever their sign, are kept together (the plain sort would split them)
+    rest = got[torch.arange(V)[(torch.arange(V) != 11) & (torch.arange(V) != 500)]]
+    assert float(rest.min()) == float(rest.max()) and got[11] > got[500] > rest[0] >= 0
+    assert bool((got > 0).all()) == bool(rest[0] > 0) and want[11] > 0
+
+
 def test_kernels_refuse_cpu_tensors(ops):
     with pytest.raises(ops.KernelError):
         ops.silu_mul(torch.zeros(2, 4))
