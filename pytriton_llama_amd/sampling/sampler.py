@@ -74,12 +74,17 @@ class Sampler:
             rs = r.params.seed if r.params.seed is not None else r.id
             params.append((r.params.temperature, r.params.top_p,
                            uniform_for(self.seed, rs, len(r.output) + ahead)))
-        p = torch.tensor(params, dtype=torch.float32).t().contiguous().to(logits.device)
+        # (through pinned memory, without waiting: the step whose logits these are may still run)
+        p = torch.tensor(params, dtype=torch.float32).t().contiguous()
+        if logits.is_cuda:
+            p = p.pin_memory().to(logits.device, non_blocking=True)
         if len(drawn) == R:
             return ops.sample_top_p(logits, p[0], p[1], p[2])
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-        gi = torch.tensor(greedy, dtype=torch.int64, device=logits.device)
-        di = torch.tensor(drawn, dtype=torch.int64, device=logits.device)
+        rows = torch.tensor(greedy + drawn, dtype=torch.int64)
+        if logits.is_cuda:
+            rows = rows.pin_memory().to(logits.device, non_blocking=True)
+        gi, di = rows[:len(greedy)], rows[len(greedy):]
         out.index_copy_(0, gi, ops.argmax(logits.index_select(0, gi)))
         out.index_copy_(0, di, ops.sample_top_p(logits.index_select(0, di), p[0], p[1], p[2]))
         return out
