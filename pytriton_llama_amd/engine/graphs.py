@@ -30,6 +30,7 @@ from typing import Dict, List, Sequence
 import numpy as np
 import torch
 
+from .. import ops
 from .batch import GroupContext, StepContext, StepEntry, take_pages
 
 
@@ -191,7 +192,7 @@ class DecodeGraphs:
             return logits
         if len(rows) == n:
             return logits[:n]
-        return logits.index_select(0, torch.tensor(rows, dtype=torch.int32, device=logits.device))
+        return logits.index_select(0, ops.to_device(rows, torch.int32, logits.device))
 
 
 PORTION_BUCKETS = (32, 64, 128, 256, 512, 1024)
@@ -375,4 +376,4 @@ class PortionGraphs:
         rows = [row_of[i] for i, x in enumerate(entries) if len(x.want)]
         if not rows:
             return b.logits[:0]
-        return b.logits.index_select(0, torch.tensor(rows, dtype=torch.int32, device=b.logits.device))
+        return b.logits.index_select(0, ops.to_device(rows, torch.int32, b.logits.device))

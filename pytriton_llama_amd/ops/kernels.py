@@ -46,6 +46,16 @@ def _stream():
     return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
 
 
+def to_device(values, dtype: torch.dtype, device) -> torch.Tensor:
+    """A short list of numbers as a device tensor, through pinned memory and without a wait
+    (torch.tensor(..., device=...) copies from pageable memory and blocks the host until the
+    stream has come that far, which undoes any step launched ahead)."""
+    t = torch.tensor(values, dtype=dtype)
+    if torch.device(device).type == "cpu":
+        return t
+    return t.pin_memory().to(device, non_blocking=True)
+
+
 def _check(code: int, what: str) -> None:
     if code == 0:
         return

@@ -39,7 +39,7 @@ class Sampler:
         if len(want) == len(requests):
             rows, toks = logits, tokens
         else:
-            idx = torch.tensor(want, dtype=torch.int32, device=logits.device)
+            idx = ops.to_device(want, torch.int32, logits.device)
             rows, toks = logits.index_select(0, idx), tokens.index_select(0, idx)
         return want, ops.token_logprob(rows, toks.contiguous())
 
@@ -47,7 +47,7 @@ class Sampler:
         """As ``logprobs_device`` for tokens on the host: a list with None for the requests that
         do not ask."""
         out = [None] * len(requests)
-        toks = torch.tensor(list(tokens), dtype=torch.int32, device=logits.device)
+        toks = ops.to_device(list(tokens), torch.int32, logits.device)
         want, lp = self.logprobs_device(logits, requests, toks)
         if want:
             for i, v in zip(want, lp.tolist()):
@@ -75,15 +75,11 @@ class Sampler:
             params.append((r.params.temperature, r.params.top_p,
                            uniform_for(self.seed, rs, len(r.output) + ahead)))
         # (through pinned memory, without waiting: the step whose logits these are may still run)
-        p = torch.tensor(params, dtype=torch.float32).t().contiguous()
-        if logits.is_cuda:
-            p = p.pin_memory().to(logits.device, non_blocking=True)
+        p = ops.to_device(list(zip(*params)), torch.float32, logits.device)
         if len(drawn) == R:
             return ops.sample_top_p(logits, p[0], p[1], p[2])
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-        rows = torch.tensor(greedy + drawn, dtype=torch.int64)
-        if logits.is_cuda:
-            rows = rows.pin_memory().to(logits.device, non_blocking=True)
+        rows = ops.to_device(greedy + drawn, torch.int64, logits.device)
         gi, di = rows[:len(greedy)], rows[len(greedy):]
         out.index_copy_(0, gi, ops.argmax(logits.index_select(0, gi)))
         out.index_copy_(0, di, ops.sample_top_p(logits.index_select(0, di), p[0], p[1], p[2]))
