@@ -42,7 +42,7 @@ class EngineConfig:
     max_model_len: int = 2048                # reference: max_seq_len
     seed: int = 0
     use_graphs: bool = True                  # replay decode-only steps, and steps that bring one
-                                             # portion of one prompt (up to 1,024 tokens), as HIP graphs
+                                             # portion of one prompt (up to 2,048 tokens), as HIP graphs
     async_decode: bool = True                # launch a decode step before the tokens of the one
                                              # before it have reached the host
 

@@ -14,7 +14,8 @@ and their logits are dropped.
 A step with one entry of several tokens (a prompt, or a portion of one: the first thing a
 request sees on an engine that is idle or only decoding) is some 150 launches that cost the
 host about 2.4 ms at 16 layers, more than the GPU needs for up to a thousand tokens. Such a
-step runs through a graph captured once per bucket of its token count (32, 64, ... 1024) and
+step runs through a graph captured once per bucket of its token count (32, 64, ... 512, then
+every 128 up to 2,048) and
 of the number of single-token entries beside it (0, 1, 2, 4, ...):
 the tokens are padded to the bucket with rows that write nothing to the cache (slot -1) and
 that no query block covers (the work lists name blocks up to the bucket's size; a block
@@ -195,8 +196,11 @@ class DecodeGraphs:
         return logits.index_select(0, ops.to_device(rows, torch.int32, logits.device))
 
 
-PORTION_BUCKETS = (32, 64, 128, 256, 512, 1024)
-MAX_PORTION_GRAPHS = 32          # pairs of (decoding rows, portion size) kept; others run eagerly
+# Token counts a portion is padded to. Up to 512 tokens a step launched kernel by kernel takes
+# the same time whatever its size (the host's), so coarse buckets lose nothing; beyond, the GPU
+# is the bound and padding costs what it adds, so the buckets are 128 apart.
+PORTION_BUCKETS = (32, 64, 128, 256, 512) + tuple(range(640, 2049, 128))
+MAX_PORTION_GRAPHS = 48          # pairs of (decoding rows, portion size) kept; others run eagerly
 
 
 class _PortionBucket:
@@ -265,7 +269,7 @@ class _PortionBucket:
 
 class PortionGraphs:
     """Steps of single-token entries (any number up to the largest decode bucket, also none)
-    and exactly one entry of 2 to 1,024 tokens with at most one wanted place."""
+    and exactly one entry of 2 to 2,048 tokens with at most one wanted place."""
 
     def __init__(self, model, manager, storage, max_model_len: int, device):
         if manager.states:
