@@ -339,19 +339,19 @@ def test_steps_launched_ahead_give_the_same_tokens(folder_b, dtype):
 def test_random_traffic_with_and_without_steps_ahead(folder_a):
     """Forty requests of random lengths arriving at random steps, greedy and sampled, some ending
     at an end-of-sequence token, with so few pages that requests are preempted: every request
-    gets the same tokens and the same finish reason whether steps are launched ahead or not, and
-    no page or slot is lost."""
+    gets the same tokens and the same finish reason whether steps are launched ahead or not and
+    whether they replay graphs or not, and no page or slot is lost."""
     from pytriton_llama_amd.config import EngineConfig
     from pytriton_llama_amd.engine import Engine, SamplingParams
     import random
     folder, page = folder_a
 
-    def run(async_decode):
+    def run(async_decode, use_graphs=True):
         rng = random.Random(11)
         g = torch.Generator().manual_seed(12)
         eng = Engine(folder, EngineConfig(dtype="float32", page_size=page, num_pages=36, max_num_seqs=6,
                                           max_num_batched_tokens=48, prefill_chunk=16, max_model_len=72,
-                                          seed=5, async_decode=async_decode))
+                                          seed=5, async_decode=async_decode, use_graphs=use_graphs))
         eng.scheduler.eos_token_ids = (7, 91, 200)
         todo, done, ahead = [], {}, 0
         for i in range(40):
@@ -380,3 +380,6 @@ def test_random_traffic_with_and_without_steps_ahead(folder_a):
     assert len(plain) == 40 and n0 == 0 and n1 > 0
     assert fast == plain
     assert {r for _, r in plain.values()} >= {"length", "eos"}
+    # and whether steps replay graphs (padded to buckets) or are launched kernel by kernel
+    eager, _, _ = run(False, use_graphs=False)
+    assert eager == plain
