@@ -32,7 +32,7 @@ def prompts_a():
 
 
 def test_greedy_generation_matches_the_plain_implementation(folder_a):
-    """BASELINE's Tiny A workload: 4 requests, prompts 5/9/13/17, 8 greedy tokens, pages of 4."""
+    """The first tiny workload: 4 requests, prompts 5/9/13/17, 8 greedy tokens, pages of 4."""
     from pytriton_llama_amd.generate import GenerateText
     folder, page = folder_a
     cfg, w = plain_llama.read_model_folder(folder)
@@ -80,7 +80,7 @@ def test_preemption_does_not_change_greedy_output(folder_a):
 
 
 def test_seeded_temperature_sampling(folder_b):
-    """BASELINE's Tiny B workload: 3 requests, prompts 31/70/100, 12 tokens at
+    """The second tiny workload: 3 requests, prompts 31/70/100, 12 tokens at
     temperature 0.8, pages of 16, 32-token portions. The same seed gives the same
     tokens whatever the batching; another seed gives others."""
     from pytriton_llama_amd.config import EngineConfig

@@ -1,5 +1,5 @@
-"""Small Llama configurations for the tests. A and B are BASELINE's tiny shapes
-and differ in every size and option; C has an explicit head_dim that is not
+"""Small Llama configurations for the tests. A and B are two tiny shapes that
+differ in every size and option; C has an explicit head_dim that is not
 hidden/heads, a width, a feed-forward and a vocabulary that are no power of
 two, and untied weights with scaling of the other type key ("type")."""
 import copy
