@@ -79,12 +79,17 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 15, lg = lane >> 4;
   const int xor16 = 4 * (lane ^ 16), xor32 = 4 * (lane ^ 32);
-  const int head = blockIdx.y;
-  // The work list is sorted, the blocks with the most keys first. The gridDim.x workgroups of a
+  // Heads run along x, the fast index of the launch, so that workgroups started one after the
+  // other land on the eight XCDs in turn; the heads are dealt out so that XCD c gets heads
+  // c * Hq/8 .. (c+1) * Hq/8 - 1: the query heads of a kv head meet in one L2, which then holds
+  // an eighth of the keys and values instead of all of them.
+  const int head = (Hq % 8 == 0) ? (blockIdx.x % 8) * (Hq / 8) + blockIdx.x / 8 : blockIdx.x;
+  const int group_at = blockIdx.y, n_groups = gridDim.y;
+  // The work list is sorted, the blocks with the most keys first. The n_groups workgroups of a
   // head walk it as a snake: forwards in even rounds, backwards in odd ones, so that the
   // workgroup with the longest block of one round takes the shortest of the next.
   for (int round = 0;; ++round) {
-  const int item = round * gridDim.x + ((round & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x);
+  const int item = round * n_groups + ((round & 1) ? n_groups - 1 - group_at : group_at);
   if (item >= n_work) break;       // (and so is every later item of this workgroup)
   const int seq = work_seq[item];
   const int qoff = work_qoff[item];
@@ -361,7 +366,7 @@ static int launch_prefill_mfma(void* out, long out_stride, const void* q, long q
                                const int32_t* work_seq, const int32_t* work_qoff, int n_work,
                                int n_groups, int Hq, int Hkv, int page_size, int window, float scale,
                                hipStream_t stream) {
-  dim3 grid(n_groups, Hq);
+  dim3 grid(Hq, n_groups < 65535 ? n_groups : 65535);
   int page_shift = -1;
   for (int sh = 0; sh < 31; ++sh)
     if ((1 << sh) == page_size) page_shift = sh;

@@ -534,17 +534,18 @@ def _compute_units(device_index: int) -> int:
 
 def attention_prefill_mfma_plan(device: torch.device, num_heads: int, head_dim: int,
                                 blocks_of_64: int, blocks_of_128: int):
-    """(block_rows, groups) for ``attention_prefill_mfma``. As many workgroups a head as the
-    chip holds at once (three a compute unit up to head size 64, two above), so that all run
-    side by side and the snake over the sorted work list evens out the causal triangle;
-    128-row blocks (keys and values are staged half as often) only when every workgroup gets
-    at least two of them."""
+    """(block_rows, groups) for ``attention_prefill_mfma``, from sweeps on MI355X (one sequence
+    of 512 to 16,384 tokens, head sizes 64 and 128). With t = the workgroups a head can have
+    resident at once (three a compute unit up to head size 64, two above): 128-row blocks
+    (keys and values are staged half as often) once there are 1.25 t of them, 64-row blocks
+    before; a workgroup for every block while there are at most 2 t blocks (the longest start
+    first and the short ones fill in behind them), beyond that t workgroups that share the
+    sorted list as a snake, which evens out the causal triangle."""
     index = device.index if device.index is not None else torch.cuda.current_device()
     resident = _compute_units(index) * (3 if head_dim <= 64 else 2)
-    groups = max(1, resident // num_heads)
-    if blocks_of_128 >= 2 * groups:
-        return 128, groups
-    return 64, max(1, min(groups, blocks_of_64))
+    t = max(1, resident // num_heads)
+    rows, blocks = (128, blocks_of_128) if 4 * blocks_of_128 >= 5 * t else (64, blocks_of_64)
+    return rows, max(1, blocks if blocks <= 2 * t else t)
 
 
 def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,

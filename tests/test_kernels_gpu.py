@@ -475,13 +475,19 @@ def test_attention_prefill_mfma_workgroups_share_the_blocks(ops, kernel, groups)
 
 
 def test_attention_prefill_mfma_plan(ops):
-    """128-row blocks only when every workgroup gets two; never more workgroups than blocks."""
+    """128-row blocks once there are 1.25 t of them (t: workgroups a head can have resident);
+    a workgroup a block up to 2 t blocks, t workgroups beyond; never more workgroups than blocks."""
     dev = torch.device("cuda", 0)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    per_head = max(1, 3 * cus // 32)
-    assert ops.attention_prefill_mfma_plan(dev, 32, 64, 3, 2) == (64, min(3, per_head))
-    assert ops.attention_prefill_mfma_plan(dev, 32, 64, 4 * per_head, 2 * per_head) == (128, per_head)
-    assert ops.attention_prefill_mfma_plan(dev, 32, 64, 4 * per_head - 2, 2 * per_head - 1) == (64, per_head)
+    t = max(1, 3 * cus // 32)
+    plan = lambda n64, n128: ops.attention_prefill_mfma_plan(dev, 32, 64, n64, n128)
+    assert plan(3, 2) == (64, 3)
+    assert plan(2 * t, t) == (64, 2 * t)
+    assert plan(2 * t + 2, t + 1) == (64, t)
+    n128 = -(-5 * t // 4)
+    assert plan(2 * n128, n128) == (128, n128)
+    assert plan(2 * n128 - 2, n128 - 1)[0] == 64
+    assert plan(8 * t, 4 * t) == (128, t)
     assert ops.attention_prefill_mfma_plan(dev, 4 * cus, 128, 1, 1) == (64, 1)
 
 
