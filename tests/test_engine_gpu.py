@@ -1,5 +1,5 @@
 """The engine against the plain implementation under every way of cutting the
-work, in float32 and in bfloat16, for three tiny configurations."""
+work, in float32 and in bfloat16, for three tiny configurations and for some drawn at random."""
 import pytest
 import torch
 
@@ -100,3 +100,51 @@ def test_long_decoding(cases, dtype):
     got = replay(runner, steps, seqs)
     bad = first_mismatch(got, want, TOL[dtype])
     assert bad is None, bad
+
+
+def _drawn_configuration(rng):
+    """A Llama configuration with every size drawn: head sizes in steps of 16 up to 256, any
+    number of kv heads and of query heads a kv head, widths, feed-forward sizes and
+    vocabularies that are no power of two (some no multiple of 8, which the bfloat16 matrix
+    kernels refuse and the general ones take), both spellings of the scaling's type key."""
+    kv_heads = rng.choice([1, 2, 3, 5])
+    scaling = None
+    if rng.random() < 0.6:
+        scaling = {rng.choice(["rope_type", "type"]): "llama3", "factor": rng.choice([2.0, 8.0, 32.0]),
+                   "low_freq_factor": 1.0, "high_freq_factor": rng.choice([2.0, 4.0]),
+                   "original_max_position_embeddings": rng.choice([32, 64, 256])}
+    return {"architectures": ["LlamaForCausalLM"], "model_type": "llama",
+            "num_hidden_layers": rng.randint(1, 3),
+            "hidden_size": rng.choice([8 * rng.randint(4, 40), 2 * rng.randint(17, 99)]),
+            "num_attention_heads": kv_heads * rng.choice([1, 2, 3, 4, 6, 7, 8, 16]),
+            "num_key_value_heads": kv_heads,
+            "head_dim": rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256]),
+            "intermediate_size": rng.choice([8 * rng.randint(5, 60), 2 * rng.randint(21, 150)]),
+            "vocab_size": rng.choice([rng.randint(100, 2000), rng.randint(2000, 40000) | 1]),
+            "rope_theta": rng.choice([1e3, 1e4, 5e5]), "rope_scaling": scaling,
+            "rms_norm_eps": rng.choice([1e-3, 1e-5, 1e-6]), "tie_word_embeddings": rng.random() < 0.5,
+            "torch_dtype": "float32", "hidden_act": "silu", "max_position_embeddings": 4096}
+
+
+@pytest.mark.parametrize("seed", [1, 3, 10, 17, 33, 40, 48, 58])
+def test_drawn_configurations_mixed_with_page_reuse(tmp_path, gpu_device, seed):
+    """Configurations drawn at random (sizes, options, page size), five requests of 2 to 420
+    tokens in a mixed batch with so few pages that they are used again, in both dtypes."""
+    import random
+    from pytriton_llama_amd.weights import write_random_model
+    rng = random.Random(seed)
+    cfg = _drawn_configuration(rng)
+    page = rng.choice([4, 8, 16, 32, 64])
+    lengths = [rng.randint(2, 40), rng.randint(40, 140), rng.randint(140, 420), rng.randint(3, 90),
+               rng.randint(60, 300)]
+    folder = str(tmp_path)
+    write_random_model(cfg, folder, seed=seed, dtype=torch.float32, norm_std=0.1,
+                       std=0.8 / cfg["hidden_size"] ** 0.5)
+    seqs = random_sequences(cfg["vocab_size"], lengths, seed=seed)
+    steps = cuttings.mixed(seqs, seed=seed, max_live=rng.choice([2, 3, 4]))
+    pages = cuttings.max_live_tokens(steps, round_to=max(64, page)) // page
+    for dtype in DTYPES:
+        want = plain_logits(folder, seqs, dtype)
+        got = replay(load_runner(folder, dtype, page, pages, max_num_seqs=4), steps, seqs)
+        bad = first_mismatch(got, want, TOL[dtype])
+        assert bad is None, f"{cfg}, page size {page}, {dtype}: first wrong place {bad}"
