@@ -69,7 +69,10 @@ class _Bucket:
             a, k = self.spans[f"slots{g}"]
             self.np[a:a + k] = -1
         self.table_np = [self.view_np(f"table{g}").reshape(B, width) for g in range(G)]
-        self.row_owner = [[None] * B for _ in range(G)]       # (request, pages written) per row
+        # per row: (the block table whose pages the row holds, how many of them). The table is
+        # kept by identity, not by the request's name: a request that ends and comes again
+        # under the same name (after a preemption, say) has a new table with other pages.
+        self.row_owner = [[None] * B for _ in range(G)]
         empty = self.dev[:0]
         # every sequence is one 16-row block at row 0: the work list of the vector-FMA
         # attention kernel, which takes the head sizes the split-KV kernel does not
@@ -171,13 +174,13 @@ class DecodeGraphs:
                 table = group.tables[e.request]
                 slots[i] = table[pos // P] * P + pos % P
                 have = owner[i]
-                if have is not None and have[0] == e.request and have[1] <= len(table) \
+                if have is not None and have[0] is table and have[1] <= len(table) \
                         and group.spec.window is None:
                     if have[1] < len(table):
                         table_np[i, have[1]:len(table)] = table[have[1]:]
                 else:
                     table_np[i, :len(table)] = table
-                owner[i] = (e.request, len(table))
+                owner[i] = (table, len(table))
         def refresh():
             b.dev.copy_(b.host, non_blocking=True)
             if token_feed is not None:

@@ -383,3 +383,36 @@ def test_random_traffic_with_and_without_steps_ahead(folder_a):
     # and whether steps replay graphs (padded to buckets) or are launched kernel by kernel
     eager, _, _ = run(False, use_graphs=False)
     assert eager == plain
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_decode_graph_of_a_request_name_that_comes_again(folder_a, dtype):
+    """A request ends and another one comes under the same name, as long or longer (what a
+    preempted request does when it is recomputed): its pages are other ones, in another order,
+    and the decode graph's copy of the block table has to follow."""
+    from pytriton_llama_amd.config import build_model, read_config_json
+    from pytriton_llama_amd.engine.batch import StepEntry
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_weights
+    folder, page = folder_a
+    model = build_model(read_config_json(folder))
+    load_weights(model, folder, dtype, "cuda:0")
+    eager = ModelRunner(model, page, 40, 4)
+    graphed = ModelRunner(model, page, 40, 4, max_model_len=64, use_graphs=True)
+    g = torch.Generator().manual_seed(3)
+    for turn in range(5):
+        n = 20 + 4 * turn
+        toks = torch.randint(0, model.vocab_size, (n + 3,), generator=g).tolist()
+        outs = []
+        for runner in (eager, graphed):
+            if turn == 2:                       # another request holds some pages meanwhile
+                runner.step([StepEntry("other", toks[:9], [])])
+            runner.step([StepEntry("r", toks[:n], [])])
+            outs.append(torch.cat([runner.step([StepEntry("r", [t], [0])]).float().cpu()
+                                   for t in toks[n:]]))
+            runner.end("r")
+            if turn == 3:
+                runner.end("other")
+            runner.manager.check()
+        err = float((outs[0] - outs[1]).abs().max()) / float(outs[0].abs().max())
+        assert err < (1e-5 if dtype == torch.float32 else 4e-2), f"turn {turn}: {err}"

@@ -46,3 +46,33 @@ def test_wide_model_all_cuttings(wide, dtype):
         got = replay(runner, steps, seqs)
         bad = first_mismatch(got, want, TOL[dtype])
         assert bad is None, f"{dtype}: first wrong place (request, position, error) = {bad}"
+
+
+def test_wide_model_graph_replays_of_long_portions(wide):
+    """Portions of 2,048 and 1,500 tokens at the real widths, where the library picks other
+    kernels than for short ones (its stream-K product among them): a step replayed as a HIP
+    graph gives the logits of the same step launched kernel by kernel, on every replay, with
+    eager steps and synchronisations between the replays."""
+    from pytriton_llama_amd.config import build_model, read_config_json
+    from pytriton_llama_amd.engine.batch import StepEntry
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_weights
+    folder, _, _ = wide
+    model = build_model(read_config_json(folder))
+    load_weights(model, folder, torch.bfloat16, "cuda:0")
+    pages = 2 * 2112 // 16
+    eager = ModelRunner(model, 16, pages, 4)
+    graphed = ModelRunner(model, 16, pages, 4, max_model_len=2112, use_graphs=True)
+    g = torch.Generator().manual_seed(21)
+    for i, n in enumerate([2048, 2048, 1500, 2048, 1500]):
+        toks = torch.randint(0, WIDE["vocab_size"], (n + 1,), generator=g).tolist()
+        got, want = [], []
+        for runner, out in ((eager, want), (graphed, got)):
+            assert (runner.portion_graphs is not None) == (runner is graphed)
+            out.append(runner.step([StepEntry("r", toks[:n], [n - 1])]).float().cpu())
+            out.append(runner.step([StepEntry("r", toks[n:], [0])]).float().cpu())   # one decoded token
+            runner.end("r")
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            err = float((a - b).abs().max()) / float(b.abs().max())
+            assert err < 2e-2, f"replay {i} ({n} tokens): {err}"
