@@ -90,6 +90,7 @@ class _Bucket:
             num_decode_seqs=B, q_lens=[1] * B, ctx_lens=[0] * B, max_q_len=1, max_ctx_len=0)
         self.graph = None
         self.logits = None
+        self.copied = None                 # event: the last copy of ``host`` has been made
 
     def view(self, name):
         a, k = self.spans[name]
@@ -157,6 +158,10 @@ class DecodeGraphs:
         starts = take_pages(entries, m, self.model.vocab_size)
         n = len(entries)
         b = self._bucket(n)
+        # Steps are launched ahead of the GPU: the pinned buffer is written again only when
+        # its last copy to the device has been made.
+        if b.copied is not None:
+            b.copied.synchronize()
         np_ = b.view_np
         np_("token_ids")[:n] = [e.tokens[0] for e in entries]
         np_("positions")[:n] = starts
@@ -188,7 +193,9 @@ class DecodeGraphs:
         if b.graph is None:
             refresh()
             self._capture(b)
+            b.copied = torch.cuda.Event()
         refresh()
+        b.copied.record()
         b.graph.replay()
         logits = b.logits
         rows = [i for i, e in enumerate(entries) if e.want]
