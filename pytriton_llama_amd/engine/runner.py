@@ -51,7 +51,9 @@ class ModelRunner:
     @torch.inference_mode()
     def step(self, entries: Sequence[StepEntry], token_feed=None) -> torch.Tensor:
         """Float32 logits [wanted, vocab], in the order of the entries and of
-        their ``want`` lists. ``token_feed``: the entries' tokens as an int32 device tensor,
+        their ``want`` lists. With graphs on, the result of a decode-only step is the graph's
+        own buffer: it holds until the next step of this runner (work queued on the same
+        stream before that step reads it safely; copy what has to last longer). ``token_feed``: the entries' tokens as an int32 device tensor,
         for a step that replays a graph and is launched before the host knows its tokens."""
         for e in entries:
             if not self.manager.is_live(e.request):
