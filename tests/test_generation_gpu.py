@@ -378,6 +378,7 @@ def test_random_traffic_with_and_without_steps_ahead(folder_a):
     plain, n0, p0 = run(False)
     fast, n1, p1 = run(True)
     assert len(plain) == 40 and n0 == 0 and n1 > 0
+    assert p0 > 0 and p1 > 0                   # requests were preempted and recomputed
     assert fast == plain
     assert {r for _, r in plain.values()} >= {"length", "eos"}
     # and whether steps replay graphs (padded to buckets) or are launched kernel by kernel
