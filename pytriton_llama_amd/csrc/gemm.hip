@@ -178,6 +178,19 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u].v, xf[t][u].v, acc[t], 0, 0, 0);
   };
   if (kb < ke) load_w(wa, kb);
+  // what the epilogue of the first wave adds and multiplies by, asked for behind the first
+  // weights: it is there long before the sums of the waves have met
+  float res_in[4] = {0.f, 0.f, 0.f, 0.f}, nw_in[4] = {0.f, 0.f, 0.f, 0.f};
+  if (ADD_NORM && wave == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * lg + i;
+      if (ln < M && 4 * lg + i < ROWS && n < N) {
+        res_in[i] = bf16_to_float(an.residual[(size_t)ln * an.ldr + n]);
+        nw_in[i] = an.norm_w[n];
+      }
+    }
+  }
   for (int k = kb; k < ke; k += 64 * U) {
     const int k1 = k + 32 * U, k2 = k + 64 * U;
     if (k1 < ke) load_w(wb, k1);
@@ -208,9 +221,9 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
       const int n = n0 + 4 * lg + i;
       if (m < M && 4 * lg + i < ROWS && n < N) {
         // as the separate kernels do it: the product rounded to bfloat16, the sum in float32
-        const float f = round_to<bf16_t>(acc[0][i]) + bf16_to_float(an.residual[(size_t)m * an.ldr + n]);
+        const float f = round_to<bf16_t>(acc[0][i]) + res_in[i];
         an.residual[(size_t)m * an.ldr + n] = float_to_bf16(f);
-        y[(size_t)m * ldy + n] = from_float<TY>(f * an.norm_w[n]);
+        y[(size_t)m * ldy + n] = from_float<TY>(f * nw_in[i]);
         ss += f * f;
       }
     }
@@ -397,6 +410,14 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   for (int u = 0; u < 4; ++u) part[u] = (my_row && lane + 64 * u < sc.count) ? prow[lane + 64 * u] : 0.f;
   int k = kb;
   if (k < ke) load_w(k);
+  // rotation mode: the position and the cache slot that the epilogue of the first wave needs,
+  // asked for behind the first weights
+  float pos_in = 0.f;
+  int slot_in = -1;
+  if (MODE == PAIR_ROPE && wave == 0 && ln < M) {
+    pos_in = (float)rs.positions[ln];
+    slot_in = rs.slots ? rs.slots[ln] : -1;
+  }
   if (sc.partials != nullptr) {
     // the waves share the rows; a row's partial sums are added in a fixed order
     for (int m = wave; m < M; m += nwaves) {
@@ -421,6 +442,13 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     }
     k += 32 * U;
     if (k < ke) load_w(k);
+  }
+  // sines and cosines while the other waves finish
+  float sn_in[4] = {0.f, 0.f, 0.f, 0.f}, cs_in[4] = {1.f, 1.f, 1.f, 1.f};
+  if (MODE == PAIR_ROPE && wave == 0 && rs.inv_freq && group < rs.Hq + rs.Hkv) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (4 * lg + i < ROWS) sincosf(pos_in * rs.inv_freq[ROWS * tile + 4 * lg + i], &sn_in[i], &cs_in[i]);
   }
   if (nwaves > 1) {
     *reinterpret_cast<gs_f32x4_t*>(red + (((size_t)wave * 2 + 0) * 64 + lane) * 4) = acc1;
@@ -452,8 +480,7 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     const int D = rs.D, half = D >> 1;
     const int head = group;                      // 0..Hq-1: q; then Hkv k heads; then Hkv v heads
     const bool is_q = head < rs.Hq, is_k = !is_q && head < rs.Hq + rs.Hkv;
-    const float pos = (float)rs.positions[m];
-    const int slot = rs.slots ? rs.slots[m] : -1;
+    const int slot = slot_in;
     bf16_t* dst = nullptr;
     if (is_q) {
       dst = y + (size_t)m * ldy + (size_t)head * D;
@@ -470,9 +497,7 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
       // as in the unfused path, the projection is rounded to bfloat16 before the rotation
       float x1 = round_to<bf16_t>(acc1[i]), x2 = round_to<bf16_t>(acc2[i]);
       if ((is_q || is_k) && rs.inv_freq) {
-        float sn, cs;
-        sincosf(pos * rs.inv_freq[j], &sn, &cs);
-        const float o1 = x1 * cs - x2 * sn, o2 = x2 * cs + x1 * sn;
+        const float o1 = x1 * cs_in[i] - x2 * sn_in[i], o2 = x2 * cs_in[i] + x1 * sn_in[i];
         x1 = o1; x2 = o2;
       }
       dst[j] = float_to_bf16(x1);
