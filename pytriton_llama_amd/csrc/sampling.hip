@@ -36,10 +36,25 @@ argmax_partial_kernel(float* __restrict__ pv, int32_t* __restrict__ pi,
   const int lo = blockIdx.x * ARGMAX_CHUNK, hi = min(V, lo + ARGMAX_CHUNK);
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = lo + threadIdx.x; i < hi; i += 256) {
-    float v = row[i];
-    if (v != v) v = -INFINITY;
-    argmax_pick(best, bi, v, i);
+  if (hi - lo == ARGMAX_CHUNK && (reinterpret_cast<uintptr_t>(row + lo) & 15) == 0) {
+    // a whole chunk with 16-byte aligned rows: a thread's four loads are asked for at once
+    float4 v[ARGMAX_CHUNK / 1024];
+#pragma unroll
+    for (int k = 0; k < ARGMAX_CHUNK / 1024; ++k)
+      v[k] = *reinterpret_cast<const float4*>(row + lo + 4 * (threadIdx.x + 256 * k));
+#pragma unroll
+    for (int k = 0; k < ARGMAX_CHUNK / 1024; ++k) {
+      const float e[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        argmax_pick(best, bi, e[j] != e[j] ? -INFINITY : e[j], lo + 4 * (threadIdx.x + 256 * k) + j);
+    }
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+      float v = row[i];
+      if (v != v) v = -INFINITY;
+      argmax_pick(best, bi, v, i);
+    }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) argmax_pick(best, bi, __shfl_xor(best, o, 64), __shfl_xor(bi, o, 64));

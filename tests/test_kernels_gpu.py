@@ -550,15 +550,17 @@ def test_attention_page_placement_does_not_matter(ops):
     assert torch.equal(outs[0], outs[1])
 
 
-@pytest.mark.parametrize("V", [1003, 4096, 128256])
+@pytest.mark.parametrize("V", [1003, 4096, 8193, 128256])
 def test_argmax(ops, V):
     torch.manual_seed(5)
     logits = torch.randn(6, V, device="cuda")
     logits[2, 7] = logits[2, V - 100] = 50.0       # a tie goes to the lowest id, across chunks too
+    logits[3, 401] = logits[3, 402] = 70.0         # ... and inside one 16-byte load
     logits[4, V - 1] = 60.0
+    logits[1, 0] = logits[5, 9] = float("nan")     # a NaN is never the choice
     got = ops.argmax(logits).cpu()
-    want = torch.argmax(logits.cpu(), dim=-1)
-    want[2] = 7
+    want = torch.argmax(torch.nan_to_num(logits.cpu(), nan=-float("inf")), dim=-1)
+    want[2], want[3] = 7, 401
     assert got.tolist() == want.tolist()
 
 
