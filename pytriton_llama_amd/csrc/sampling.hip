@@ -68,28 +68,34 @@ argmax_partial_kernel(float* __restrict__ pv, int32_t* __restrict__ pi,
   }
 }
 
+// host_out (optional): pinned host memory that receives the choices as well, written over the
+// bus by this kernel, so that the host needs no copy after it
 __global__ void __launch_bounds__(64)
 argmax_final_kernel(int32_t* __restrict__ out, const float* __restrict__ pv,
-                    const int32_t* __restrict__ pi, int chunks) {
+                    const int32_t* __restrict__ pi, int chunks, int32_t* __restrict__ host_out) {
   float best = -INFINITY;
   int bi = 0x7fffffff;
   for (int i = threadIdx.x; i < chunks; i += 64)
     argmax_pick(best, bi, pv[(size_t)blockIdx.x * chunks + i], pi[(size_t)blockIdx.x * chunks + i]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) argmax_pick(best, bi, __shfl_xor(best, o, 64), __shfl_xor(bi, o, 64));
-  if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+  if (threadIdx.x == 0) {
+    const int choice = bi == 0x7fffffff ? 0 : bi;
+    out[blockIdx.x] = choice;
+    if (host_out != nullptr) host_out[blockIdx.x] = choice;
+  }
 }
 
 // workspace: float [R, chunks] and int32 [R, chunks], chunks = ceil(V / 4096)
 extern "C" int ptl_argmax(int32_t* out, const float* logits, int R, int V, long stride,
-                          float* ws_val, int32_t* ws_idx, hipStream_t stream) {
+                          float* ws_val, int32_t* ws_idx, int32_t* host_out, hipStream_t stream) {
   if (R <= 0) return PTL_OK;
   if (V <= 0 || stride < V || !ws_val || !ws_idx || R > 65535) return PTL_ERR_ARG;
   const int chunks = (V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
   dim3 grid(chunks, R);
   argmax_partial_kernel<<<grid, 256, 0, stream>>>(ws_val, ws_idx, logits, V, stride, chunks);
   if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
-  argmax_final_kernel<<<R, 64, 0, stream>>>(out, ws_val, ws_idx, chunks);
+  argmax_final_kernel<<<R, 64, 0, stream>>>(out, ws_val, ws_idx, chunks, host_out);
   return ptl_launch_status();
 }
 

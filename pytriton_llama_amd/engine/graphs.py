@@ -187,9 +187,9 @@ class DecodeGraphs:
                     table_np[i, :len(table)] = table
                 owner[i] = (table, len(table))
         def refresh():
-            b.dev.copy_(b.host, non_blocking=True)
-            if token_feed is not None:
-                b.view("token_ids")[:n].copy_(token_feed[:n], non_blocking=True)
+            # one short kernel reads the pinned buffer and, for a step launched ahead, the
+            # tokens the step before left on the device
+            ops.stage_step(b.dev, b.host, token_feed, b.spans["token_ids"][0], n)
         if b.graph is None:
             refresh()
             self._capture(b)

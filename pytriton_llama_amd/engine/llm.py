@@ -135,13 +135,10 @@ class Engine:
         replayed = self.runner.replays(entries)
         logits = self.runner.step(entries, before.tokens if before is not None else None)
         ahead = 1 if before is not None else 0
-        tokens = self.sampler.sample_device(logits, samplers, ahead)
-        want_lp, lps = self.sampler.logprobs_device(logits, samplers, tokens)
         host_tokens, host_lps = self._pinned[self._turn % len(self._pinned)]
         self._turn += 1
-        n = len(samplers)
-        if n:
-            host_tokens[:n].copy_(tokens, non_blocking=True)
+        tokens = self.sampler.sample_device(logits, samplers, ahead, host_tokens)
+        want_lp, lps = self.sampler.logprobs_device(logits, samplers, tokens)
         if want_lp:
             host_lps[:len(want_lp)].copy_(lps, non_blocking=True)
         done = torch.cuda.Event()

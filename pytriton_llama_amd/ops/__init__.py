@@ -6,4 +6,4 @@ from .kernels import (PROBE_MFMA_FLOPS_PER_ITER, KernelError, RowScale, add_rmsn
                       gemm_library, gemm_library_fits, gemm_nt, gemm_skinny, gemm_skinny_add_norm, gemm_skinny_add_norm_fits,
                       gemm_skinny_fits, probe_mfma, probe_stream_read, qkv_rope_store, qkv_rope_store_fits,
                       rope_store, row_scale,
-                      sample_top_p, silu_mul, to_device, token_logprob)
+                      sample_top_p, silu_mul, stage_step, to_device, token_logprob)

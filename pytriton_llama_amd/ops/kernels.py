@@ -85,6 +85,27 @@ def embedding(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def stage_step(dst: torch.Tensor, src: torch.Tensor, tokens: Optional[torch.Tensor] = None,
+               tok_at: int = 0, n_tok: int = 0) -> None:
+    """dst (int32, device) <- src (int32, pinned host memory of the same length), read by a
+    kernel over the bus; dst[tok_at : tok_at + n_tok] <- tokens (int32, device) when given."""
+    _need_gpu(dst)
+    if src.is_cuda or not src.is_pinned():
+        raise KernelError("stage_step: the source must be pinned host memory")
+    if (dst.dtype != torch.int32 or src.dtype != torch.int32 or dst.numel() != src.numel()
+            or not dst.is_contiguous() or not src.is_contiguous()):
+        raise KernelError("stage_step: two contiguous int32 buffers of one length")
+    if tokens is not None:
+        _need_gpu(tokens)
+        _i32(tokens, "tokens")
+        if not (0 <= tok_at and 0 <= n_tok <= tokens.numel() and tok_at + n_tok <= dst.numel()):
+            raise KernelError("stage_step: the tokens do not fit where they are to go")
+    lib = library.load("embedding")
+    _check(lib.ptl_stage_step(_ptr(dst), ctypes.c_void_p(src.data_ptr()), dst.numel(),
+                              _ptr(tokens) if tokens is not None else None, int(tok_at),
+                              int(n_tok) if tokens is not None else 0, _stream()), "stage_step")
+
+
 def add_rmsnorm(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor,
                 eps: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = rmsnorm(x + residual) * weight; ``residual`` (if given) is replaced
@@ -585,19 +606,24 @@ def attention_prefill_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
         int(window), ctypes.c_float(scale), _stream()), "attention_prefill_mfma")
 
 
-def argmax(logits: torch.Tensor) -> torch.Tensor:
-    """Greedy token per row of float32 logits [R, V]; ties go to the lowest id."""
+def argmax(logits: torch.Tensor, host_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Greedy token per row of float32 logits [R, V]; ties go to the lowest id. ``host_out``:
+    pinned int32 host memory (at least R long) that the kernel fills as well, over the bus;
+    it holds the choices once the kernel has ended (an event after it, say)."""
     _need_gpu(logits)
     if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelError("argmax: logits must be float32 [R, V] with dense rows")
     R, V = logits.shape
+    if host_out is not None and (host_out.is_cuda or not host_out.is_pinned() or host_out.dtype != torch.int32
+                                 or not host_out.is_contiguous() or host_out.numel() < R):
+        raise KernelError("argmax: host_out must be pinned int32 host memory with a place for every row")
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     chunks = -(-V // 4096)
     ws_val = torch.empty((R, chunks), dtype=torch.float32, device=logits.device)
     ws_idx = torch.empty((R, chunks), dtype=torch.int32, device=logits.device)
     lib = library.load("sampling")
     _check(lib.ptl_argmax(_ptr(out), _ptr(logits), R, V, ctypes.c_long(logits.stride(0)),
-                          _ptr(ws_val), _ptr(ws_idx), _stream()), "argmax")
+                          _ptr(ws_val), _ptr(ws_idx), _ptr(host_out), _stream()), "argmax")
     return out
 
 

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import hashlib
 import struct
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
@@ -27,6 +27,7 @@ class Sampler:
 
     def __init__(self, seed: int = 0):
         self.seed = int(seed)
+        self._wrote_host = False
 
     def logprobs_device(self, logits: torch.Tensor, requests: Sequence[Request],
                         tokens: torch.Tensor):
@@ -54,19 +55,31 @@ class Sampler:
                 out[i] = v
         return out
 
-    def sample_device(self, logits: torch.Tensor, requests: Sequence[Request],
-                      ahead: int = 0) -> torch.Tensor:
+    def sample_device(self, logits: torch.Tensor, requests: Sequence[Request], ahead: int = 0,
+                      host_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """logits float32 [R, V], row i for requests[i]; R token ids, int32, on the device (no
         wait for them). ``ahead``: how many tokens of each request are still on their way and
-        not in its output list yet (they count for the index of the random number)."""
+        not in its output list yet (they count for the index of the random number).
+        ``host_out``: pinned int32 host memory that receives the tokens too (when every row is
+        greedy the arg-max kernel writes them there itself, otherwise a copy is queued); it
+        holds them once the work queued here has ended."""
+        tokens = self._sample_device(logits, requests, ahead, host_out)
+        if host_out is not None and tokens is not None and not self._wrote_host:
+            host_out[:len(requests)].copy_(tokens, non_blocking=True)
+        return tokens
+
+    def _sample_device(self, logits, requests, ahead, host_out):
+        self._wrote_host = False
         R = len(requests)
         if logits.shape[0] != R:
             raise ValueError(f"{logits.shape[0]} rows of logits for {R} requests")
         if R == 0:
+            self._wrote_host = True
             return torch.empty((0,), dtype=torch.int32, device=logits.device)
         greedy = [i for i, r in enumerate(requests) if r.params.temperature == 0]
         if len(greedy) == R:
-            return ops.argmax(logits)
+            self._wrote_host = host_out is not None
+            return ops.argmax(logits, host_out)
         drawn = [i for i, r in enumerate(requests) if r.params.temperature != 0]
         params = []
         for i in drawn:

@@ -30,6 +30,25 @@ def test_embedding(ops, dtype):
     assert torch.equal(ops.embedding(table, ids), table[ids.long()])
 
 
+def test_stage_step(ops):
+    """The tables of a replayed step go from pinned host memory to the device buffer by a
+    kernel; tokens that are still on the device take their places among them."""
+    host = torch.arange(1000, 1000 + 777, dtype=torch.int32).pin_memory()
+    dev = torch.zeros(777, dtype=torch.int32, device="cuda")
+    ops.stage_step(dev, host)
+    assert torch.equal(dev.cpu(), host)
+    tokens = torch.tensor([7, 8, 9, 10], dtype=torch.int32, device="cuda")
+    host[:] = torch.arange(777, dtype=torch.int32)
+    ops.stage_step(dev, host, tokens, 300, 3)
+    want = host.clone()
+    want[300:303] = torch.tensor([7, 8, 9], dtype=torch.int32)
+    assert torch.equal(dev.cpu(), want)
+    with pytest.raises(ops.KernelError):
+        ops.stage_step(dev, torch.zeros(777, dtype=torch.int32))          # not pinned
+    with pytest.raises(ops.KernelError):
+        ops.stage_step(dev, host, tokens, 775, 4)                         # past the end
+
+
 @pytest.mark.parametrize("dtype", DT, ids=IDS)
 @pytest.mark.parametrize("shape", [(5, 72), (3, 2048), (2, 5000), (1, 16)])
 def test_add_rmsnorm(ops, dtype, shape):
@@ -562,6 +581,11 @@ def test_argmax(ops, V):
     want = torch.argmax(torch.nan_to_num(logits.cpu(), nan=-float("inf")), dim=-1)
     want[2], want[3] = 7, 401
     assert got.tolist() == want.tolist()
+    # the kernel can leave the choices in pinned host memory as well
+    host = torch.full((8,), -1, dtype=torch.int32).pin_memory()
+    again = ops.argmax(logits, host_out=host)
+    torch.cuda.synchronize()
+    assert again.cpu().tolist() == want.tolist() and host.tolist() == want.tolist() + [-1, -1]
 
 
 def test_sample_top_p_distribution(ops):
