@@ -116,6 +116,44 @@ union GsFrag {
   gs_bf16x8_t v;
 };
 
+// x for few rows, with fewer load instructions. The MFMA takes x^T as B: lane (ln, lg) holds
+// row ln of x, 8 elements of k-group lg, for one block of 32 k. With M <= XR rows (XR = 1, 2, 4,
+// 8) only the lanes ln < XR of a block matter, so one load instruction fetches 16 / XR blocks at
+// once: lane ln asks for row ln % XR of block ln / XR. Block j then reaches the lanes ln < XR by
+// a shift of XR * j lanes inside the rows of 16 lanes (DPP row_shl, no memory and no LDS). The
+// other lanes of a shifted fragment hold rows of other blocks or zeros: they feed result
+// columns m >= XR >= M, which are never stored. Halving the load instructions of x at 8 rows
+// took 60 us off a decode step of 1.15 ms: the instructions count, not the bytes.
+template <int SH>
+__device__ __forceinline__ uint4 gs_from_lane_up(uint4 v) {      // lane i <- lane i + SH of its row
+  constexpr int ctrl = 0x100 + SH;                               // row_shl:SH
+  uint4 r;
+  r.x = __builtin_amdgcn_update_dpp(0, (int)v.x, ctrl, 0xf, 0xf, true);
+  r.y = __builtin_amdgcn_update_dpp(0, (int)v.y, ctrl, 0xf, 0xf, true);
+  r.z = __builtin_amdgcn_update_dpp(0, (int)v.z, ctrl, 0xf, 0xf, true);
+  r.w = __builtin_amdgcn_update_dpp(0, (int)v.w, ctrl, 0xf, 0xf, true);
+  return r;
+}
+__device__ __forceinline__ uint4 gs_from_lane_up_by(uint4 v, int sh) {   // sh: a constant after unrolling
+  switch (sh) {
+    case 1: return gs_from_lane_up<1>(v);
+    case 2: return gs_from_lane_up<2>(v);
+    case 3: return gs_from_lane_up<3>(v);
+    case 4: return gs_from_lane_up<4>(v);
+    case 5: return gs_from_lane_up<5>(v);
+    case 6: return gs_from_lane_up<6>(v);
+    case 7: return gs_from_lane_up<7>(v);
+    case 8: return gs_from_lane_up<8>(v);
+    case 10: return gs_from_lane_up<10>(v);
+    case 12: return gs_from_lane_up<12>(v);
+    case 14: return gs_from_lane_up<14>(v);
+    default: return v;
+  }
+}
+// blocks of 32 k that one load instruction fetches with XR rows a block (at most U of them)
+template <int XR, int U> struct GsPack { static constexpr int P = (16 / XR < U) ? 16 / XR : U; };
+static int gs_rows_of(int M) { return M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16; }
+
 // The follow-up of a product whose result is added to the residual stream and normalised
 // (ptl_gemm_skinny_add_norm_bf16). The normalisation needs the whole row, which no workgroup
 // has, so the product's kernel does what it can see: s = round_bf16(x W^T) + residual, the
@@ -132,7 +170,8 @@ struct AddNormArgs {
 // ROWS: weight rows a workgroup owns: 16 fill the MFMA tile; 8 (half the tile idle) give twice
 // the workgroups when N is so small that 16-row tiles would leave CUs without work.
 // ADD_NORM: the epilogue described at AddNormArgs (MT = 1, bfloat16 output).
-template <int MT, int U, int ROWS, typename TY, bool ADD_NORM = false>
+// XR: rows of x a packed load takes per block (see gs_from_lane_up); 16: no packing.
+template <int MT, int U, int ROWS, typename TY, bool ADD_NORM = false, int XR = 16>
 __global__ void __launch_bounds__(1024)
 gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                    int M, int N, int K, long ldx, long ldy, int k_per_wave, AddNormArgs an) {
@@ -142,9 +181,13 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
   const int n0 = blockIdx.x * ROWS;
   const bool wrow = ln < ROWS;
   const bf16_t* wp = w + (size_t)min(n0 + min(ln, ROWS - 1), N - 1) * K + 8 * lg;
+  static_assert(XR == 16 || MT == 1, "packed loads of x are for one tile of rows");
+  constexpr int P = GsPack<XR, U>::P;          // blocks a load instruction of x fetches
+  const int xrow = ln % XR, xblock = ln / XR;
   const bf16_t* xp[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) xp[t] = x + (size_t)min(16 * t + ln, M - 1) * ldx + 8 * lg;
+  for (int t = 0; t < MT; ++t)
+    xp[t] = x + (size_t)min(16 * t + xrow, M - 1) * ldx + 8 * lg + 32 * (xblock < P ? xblock : 0);
   gs_f32x4_t acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = gs_f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -154,7 +197,7 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
   // Two sets of weight registers: the loads of the next 32 U columns are under way while
   // this set is multiplied, and a wave with at most 64 U columns has asked for all of its
   // weights before it waits for any. x, which lies in L2, is fetched as it is needed.
-  GsFrag wa[U], wb[U], xf[MT][U];
+  GsFrag wa[U], wb[U], xf[MT][U / P];
   auto load_w = [&](GsFrag (&wf)[U], int k) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -164,18 +207,21 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
   };
   auto multiply = [&](GsFrag (&wf)[U], int k) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const bool ok = k + 32 * u + 8 * lg < ke;
+    for (int v = 0; v < U / P; ++v) {
+      const bool ok = xblock < P && k + 32 * (v * P + xblock) + 8 * lg < ke;
 #pragma unroll
       for (int t = 0; t < MT; ++t)   // columns past the last row of x are never stored: no load
-        xf[t][u].u = (ok && 16 * t + ln < M) ? *reinterpret_cast<const uint4*>(xp[t] + k + 32 * u)
-                                             : make_uint4(0, 0, 0, 0);
+        xf[t][v].u = (ok && 16 * t + xrow < M) ? *reinterpret_cast<const uint4*>(xp[t] + k + 32 * v * P)
+                                               : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u].v, xf[t][u].v, acc[t], 0, 0, 0);
+      for (int t = 0; t < MT; ++t) {
+        GsFrag f;
+        f.u = gs_from_lane_up_by(xf[t][u / P].u, XR * (u % P));
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u].v, f.v, acc[t], 0, 0, 0);
+      }
   };
   if (kb < ke) load_w(wa, kb);
   // what the epilogue of the first wave adds and multiplies by, asked for behind the first
@@ -258,17 +304,28 @@ static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int 
   if (waves < 4 && K >= 1024) waves = 4;
   int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * MT * 64 * 4 * sizeof(float) : 0;
+  const int xr = MT == 1 ? gs_rows_of(M) : 16;
+#define GO(TY, AN, XR, args)                                                                         \
+  gemm_skinny_kernel<(XR == 16 ? MT : 1), U, ROWS, TY, AN, XR><<<blocks, waves * 64, lds, stream>>>(   \
+      (TY*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, args)
+#define BY_ROWS(TY, AN, args)                                                                        \
+  switch (xr) {                                                                                      \
+    case 1: GO(TY, AN, 1, args); break;                                                              \
+    case 2: GO(TY, AN, 2, args); break;                                                              \
+    case 4: GO(TY, AN, 4, args); break;                                                              \
+    case 8: GO(TY, AN, 8, args); break;                                                              \
+    default: GO(TY, AN, 16, args); break;                                                            \
+  }
   if (an != nullptr) {
     if (MT != 1 || out_dtype != PTL_DTYPE_BF16) return PTL_ERR_ARG;
-    gemm_skinny_kernel<1, U, ROWS, bf16_t, true><<<blocks, waves * 64, lds, stream>>>(
-        (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, *an);
+    BY_ROWS(bf16_t, true, *an)
   } else if (out_dtype == PTL_DTYPE_F32) {
-    gemm_skinny_kernel<MT, U, ROWS, float><<<blocks, waves * 64, lds, stream>>>(
-        (float*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, AddNormArgs{});
+    BY_ROWS(float, false, AddNormArgs{})
   } else {
-    gemm_skinny_kernel<MT, U, ROWS, bf16_t><<<blocks, waves * 64, lds, stream>>>(
-        (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, AddNormArgs{});
+    BY_ROWS(bf16_t, false, AddNormArgs{})
   }
+#undef BY_ROWS
+#undef GO
   return ptl_launch_status();
 }
 
@@ -355,7 +412,7 @@ struct RowScaleArgs {
   float inv_n, eps;
 };
 
-template <int MODE, int U, int ROWS>
+template <int MODE, int U, int ROWS, int XR>
 __global__ void __launch_bounds__(1024)
 gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                  int M, int N_out, int K, long ldx, long ldy, int k_per_wave, int pair_offset,
@@ -375,12 +432,14 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   const bool wrow = ln < ROWS;
   const bf16_t* wp1 = w + (size_t)(r1 + min(ln, ROWS - 1)) * K + 8 * lg;
   const bf16_t* wp2 = w + (size_t)(r2 + min(ln, ROWS - 1)) * K + 8 * lg;
-  const bf16_t* xp = x + (size_t)min(ln, M - 1) * ldx + 8 * lg;
+  constexpr int P = GsPack<XR, U>::P;          // blocks a load instruction of x fetches
+  const int xrow = ln % XR, xblock = ln / XR;
+  const bf16_t* xp = x + (size_t)min(xrow, M - 1) * ldx + 8 * lg + 32 * (xblock < P ? xblock : 0);
   gs_f32x4_t acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
 
   const int kb = wave * k_per_wave;
   const int ke = min(K, kb + k_per_wave);
-  GsFrag w1[U], w2[U], xf[U];
+  GsFrag w1[U], w2[U], xf[U / P];
   auto load_w = [&](int k) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -391,9 +450,9 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   };
   auto load_x = [&](int k) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const bool ok = k + 32 * u + 8 * lg < ke && ln < M;
-      xf[u].u = ok ? *reinterpret_cast<const uint4*>(xp + k + 32 * u) : make_uint4(0, 0, 0, 0);
+    for (int v = 0; v < U / P; ++v) {
+      const bool ok = xblock < P && k + 32 * (v * P + xblock) + 8 * lg < ke && xrow < M;
+      xf[v].u = ok ? *reinterpret_cast<const uint4*>(xp + k + 32 * v * P) : make_uint4(0, 0, 0, 0);
     }
   };
   // The first weights set out before anything else: they come from HBM and are what the
@@ -437,8 +496,10 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     load_x(k);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, xf[u].v, acc1, 0, 0, 0);
-      acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2[u].v, xf[u].v, acc2, 0, 0, 0);
+      GsFrag f;
+      f.u = gs_from_lane_up_by(xf[u / P].u, XR * (u % P));
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u].v, f.v, acc1, 0, 0, 0);
+      acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2[u].v, f.v, acc2, 0, 0, 0);
     }
     k += 32 * U;
     if (k < ke) load_w(k);
@@ -528,9 +589,17 @@ extern "C" int ptl_gate_up_silu_bf16(void* out, const void* x, const void* w, in
   const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
   RopeStoreArgs none = {};
-  gemm_pair_kernel<PAIR_SILU, 8, 16><<<blocks, waves * 64, lds, stream>>>(
-      (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, I, K, ldx, I, k_per_wave, I, blocks, 0, none,
-      sc);
+#define GO(XR)                                                                                        \
+  gemm_pair_kernel<PAIR_SILU, 8, 16, XR><<<blocks, waves * 64, lds, stream>>>(                        \
+      (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, I, K, ldx, I, k_per_wave, I, blocks, 0, none, sc)
+  switch (gs_rows_of(M)) {
+    case 1: GO(1); break;
+    case 2: GO(2); break;
+    case 4: GO(4); break;
+    case 8: GO(8); break;
+    default: GO(16); break;
+  }
+#undef GO
   return ptl_launch_status();
 }
 
@@ -555,13 +624,20 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
   const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
   RopeStoreArgs rs = {positions, inv_freq, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, Hq, Hkv, D, page_size};
-  if (small)
-    gemm_pair_kernel<PAIR_ROPE, 8, 8><<<blocks, waves * 64, lds, stream>>>(
-        (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,
-        tiles, D, rs, sc);
-  else
-    gemm_pair_kernel<PAIR_ROPE, 8, 16><<<blocks, waves * 64, lds, stream>>>(
-        (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,
-        tiles, D, rs, sc);
+#define GO(ROWS, XR)                                                                                  \
+  gemm_pair_kernel<PAIR_ROPE, 8, ROWS, XR><<<blocks, waves * 64, lds, stream>>>(                      \
+      (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,  \
+      tiles, D, rs, sc)
+#define BY_ROWS(ROWS)                                                                                 \
+  switch (gs_rows_of(M)) {                                                                            \
+    case 1: GO(ROWS, 1); break;                                                                       \
+    case 2: GO(ROWS, 2); break;                                                                       \
+    case 4: GO(ROWS, 4); break;                                                                       \
+    case 8: GO(ROWS, 8); break;                                                                       \
+    default: GO(ROWS, 16); break;                                                                     \
+  }
+  if (small) { BY_ROWS(8) } else { BY_ROWS(16) }
+#undef BY_ROWS
+#undef GO
   return ptl_launch_status();
 }

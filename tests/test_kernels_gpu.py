@@ -105,7 +105,9 @@ def test_gemm_nt(ops, dtype, mnk):
                                  (33, 16, 8192), (64, 1000, 64), (8, 2048, 8192), (5, 130, 2056),
                                  # a W wide enough for the streaming form: tiles past the end, K with a
                                  # partial last batch, one row and sixteen
-                                 (1, 16384, 256), (8, 20003, 328), (16, 17000, 2048), (3, 40001, 72)])
+                                 (1, 16384, 256), (8, 20003, 328), (16, 17000, 2048), (3, 40001, 72),
+                                 # every way of packing the loads of x: 1, 2, 4, 8 rows a block, and none
+                                 (2, 520, 264), (4, 136, 1032), (6, 264, 520), (9, 72, 296), (2, 4112, 2048)])
 def test_gemm_skinny(ops, out_dtype, mnk):
     M, N, K = mnk
     torch.manual_seed(7)
