@@ -117,8 +117,8 @@ union GsFrag {
 };
 
 // x for few rows, with fewer load instructions. The MFMA takes x^T as B: lane (ln, lg) holds
-// row ln of x, 8 elements of k-group lg, for one block of 32 k. With M <= XR rows (XR = 1, 2, 4,
-// 8) only the lanes ln < XR of a block matter, so one load instruction fetches 16 / XR blocks at
+// row ln of x, 8 elements of k-group lg, for one block of 32 k. With M <= XR rows (XR = 4 or 8)
+// only the lanes ln < XR of a block matter, so one load instruction fetches 16 / XR blocks at
 // once: lane ln asks for row ln % XR of block ln / XR. Block j then reaches the lanes ln < XR by
 // a shift of XR * j lanes inside the rows of 16 lanes (DPP row_shl, no memory and no LDS). The
 // other lanes of a shifted fragment hold rows of other blocks or zeros: they feed result
@@ -136,23 +136,16 @@ __device__ __forceinline__ uint4 gs_from_lane_up(uint4 v) {      // lane i <- la
 }
 __device__ __forceinline__ uint4 gs_from_lane_up_by(uint4 v, int sh) {   // sh: a constant after unrolling
   switch (sh) {
-    case 1: return gs_from_lane_up<1>(v);
-    case 2: return gs_from_lane_up<2>(v);
-    case 3: return gs_from_lane_up<3>(v);
     case 4: return gs_from_lane_up<4>(v);
-    case 5: return gs_from_lane_up<5>(v);
-    case 6: return gs_from_lane_up<6>(v);
-    case 7: return gs_from_lane_up<7>(v);
     case 8: return gs_from_lane_up<8>(v);
-    case 10: return gs_from_lane_up<10>(v);
     case 12: return gs_from_lane_up<12>(v);
-    case 14: return gs_from_lane_up<14>(v);
     default: return v;
   }
 }
 // blocks of 32 k that one load instruction fetches with XR rows a block (at most U of them)
 template <int XR, int U> struct GsPack { static constexpr int P = (16 / XR < U) ? 16 / XR : U; };
-static int gs_rows_of(int M) { return M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16; }
+// (measured: packing finer than four rows a block, for one or two rows, gains nothing more)
+static int gs_rows_of(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
 // The follow-up of a product whose result is added to the residual stream and normalised
 // (ptl_gemm_skinny_add_norm_bf16). The normalisation needs the whole row, which no workgroup
@@ -310,8 +303,6 @@ static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int 
       (TY*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, args)
 #define BY_ROWS(TY, AN, args)                                                                        \
   switch (xr) {                                                                                      \
-    case 1: GO(TY, AN, 1, args); break;                                                              \
-    case 2: GO(TY, AN, 2, args); break;                                                              \
     case 4: GO(TY, AN, 4, args); break;                                                              \
     case 8: GO(TY, AN, 8, args); break;                                                              \
     default: GO(TY, AN, 16, args); break;                                                            \
@@ -593,8 +584,6 @@ extern "C" int ptl_gate_up_silu_bf16(void* out, const void* x, const void* w, in
   gemm_pair_kernel<PAIR_SILU, 8, 16, XR><<<blocks, waves * 64, lds, stream>>>(                        \
       (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, I, K, ldx, I, k_per_wave, I, blocks, 0, none, sc)
   switch (gs_rows_of(M)) {
-    case 1: GO(1); break;
-    case 2: GO(2); break;
     case 4: GO(4); break;
     case 8: GO(8); break;
     default: GO(16); break;
@@ -630,8 +619,6 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
       tiles, D, rs, sc)
 #define BY_ROWS(ROWS)                                                                                 \
   switch (gs_rows_of(M)) {                                                                            \
-    case 1: GO(ROWS, 1); break;                                                                       \
-    case 2: GO(ROWS, 2); break;                                                                       \
     case 4: GO(ROWS, 4); break;                                                                       \
     case 8: GO(ROWS, 8); break;                                                                       \
     default: GO(ROWS, 16); break;                                                                     \
