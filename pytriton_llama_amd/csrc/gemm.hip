@@ -220,13 +220,26 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
   // what the epilogue of the first wave adds and multiplies by, asked for behind the first
   // weights: it is there long before the sums of the waves have met
   float res_in[4] = {0.f, 0.f, 0.f, 0.f}, nw_in[4] = {0.f, 0.f, 0.f, 0.f};
-  if (ADD_NORM && wave == 0) {
+  // a lane's four columns as one access each where strides and pointers allow it
+  const bool four = (N & 3) == 0 && (ldy & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
+                    (!ADD_NORM || ((an.ldr & 3) == 0 && (reinterpret_cast<uintptr_t>(an.residual) & 7) == 0 &&
+                                   (reinterpret_cast<uintptr_t>(an.norm_w) & 15) == 0));
+  if (ADD_NORM && wave == 0 && ln < M && 4 * lg < ROWS && n0 + 4 * lg < N) {
+    if (four) {
+      union { uint2 u; bf16_t e[4]; } r;
+      r.u = *reinterpret_cast<const uint2*>(an.residual + (size_t)ln * an.ldr + n0 + 4 * lg);
+      const float4 w4 = *reinterpret_cast<const float4*>(an.norm_w + n0 + 4 * lg);
+      nw_in[0] = w4.x; nw_in[1] = w4.y; nw_in[2] = w4.z; nw_in[3] = w4.w;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + 4 * lg + i;
-      if (ln < M && 4 * lg + i < ROWS && n < N) {
-        res_in[i] = bf16_to_float(an.residual[(size_t)ln * an.ldr + n]);
-        nw_in[i] = an.norm_w[n];
+      for (int i = 0; i < 4; ++i) res_in[i] = bf16_to_float(r.e[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 4 * lg + i;
+        if (n < N) {
+          res_in[i] = bf16_to_float(an.residual[(size_t)ln * an.ldr + n]);
+          nw_in[i] = an.norm_w[n];
+        }
       }
     }
   }
@@ -255,15 +268,30 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
   if (ADD_NORM) {
     const int m = ln;
     float ss = 0.f;
+    if (four && sizeof(TY) == 2) {
+      if (m < M && 4 * lg < ROWS && n0 + 4 * lg < N) {
+        union { uint2 u; bf16_t e[4]; } r, o;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + 4 * lg + i;
-      if (m < M && 4 * lg + i < ROWS && n < N) {
-        // as the separate kernels do it: the product rounded to bfloat16, the sum in float32
-        const float f = round_to<bf16_t>(acc[0][i]) + res_in[i];
-        an.residual[(size_t)m * an.ldr + n] = float_to_bf16(f);
-        y[(size_t)m * ldy + n] = from_float<TY>(f * nw_in[i]);
-        ss += f * f;
+        for (int i = 0; i < 4; ++i) {
+          // as the separate kernels do it: the product rounded to bfloat16, the sum in float32
+          const float f = round_to<bf16_t>(acc[0][i]) + res_in[i];
+          r.e[i] = float_to_bf16(f);
+          o.e[i] = float_to_bf16(f * nw_in[i]);
+          ss += f * f;
+        }
+        *reinterpret_cast<uint2*>(an.residual + (size_t)m * an.ldr + n0 + 4 * lg) = r.u;
+        *reinterpret_cast<uint2*>(reinterpret_cast<bf16_t*>(y) + (size_t)m * ldy + n0 + 4 * lg) = o.u;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 4 * lg + i;
+        if (m < M && 4 * lg + i < ROWS && n < N) {
+          const float f = round_to<bf16_t>(acc[0][i]) + res_in[i];
+          an.residual[(size_t)m * an.ldr + n] = float_to_bf16(f);
+          y[(size_t)m * ldy + n] = from_float<TY>(f * nw_in[i]);
+          ss += f * f;
+        }
       }
     }
     ss += __shfl_xor(ss, 16, 64);
@@ -275,6 +303,20 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
   for (int t = 0; t < MT; ++t) {
     const int m = 16 * t + ln;
     if (m >= M) continue;
+    if (four) {
+      if (4 * lg < ROWS && n0 + 4 * lg < N) {
+        TY* at = y + (size_t)m * ldy + n0 + 4 * lg;
+        if (sizeof(TY) == 4) {
+          *reinterpret_cast<float4*>(at) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+        } else {
+          union { uint2 u; bf16_t e[4]; } o;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o.e[i] = float_to_bf16(acc[t][i]);
+          *reinterpret_cast<uint2*>(at) = o.u;
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int n = n0 + 4 * lg + i;
@@ -521,12 +563,21 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   }
   if (m >= M) return;
   if (MODE == PAIR_SILU) {
+    union { uint2 u; bf16_t e[4]; } o;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int c = r1 + 4 * lg + i;
       // the gate and up products are rounded to bfloat16 as the unfused path stores them
       const float g = round_to<bf16_t>(acc1[i]), u = round_to<bf16_t>(acc2[i]);
-      if (4 * lg + i < ROWS && c < N_out) y[(size_t)m * ldy + c] = float_to_bf16(g / (1.0f + expf(-g)) * u);
+      o.e[i] = float_to_bf16(g / (1.0f + expf(-g)) * u);
+    }
+    const int c0 = r1 + 4 * lg;
+    if ((N_out & 3) == 0 && (ldy & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 7) == 0) {
+      // a lane's four columns as one 8-byte store
+      if (4 * lg < ROWS && c0 < N_out) *reinterpret_cast<uint2*>(y + (size_t)m * ldy + c0) = o.u;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (4 * lg + i < ROWS && c0 + i < N_out) y[(size_t)m * ldy + c0 + i] = o.e[i];
     }
   } else {
     const int D = rs.D, half = D >> 1;
