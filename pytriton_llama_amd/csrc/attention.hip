@@ -523,7 +523,6 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
   constexpr int VCH = 16 * CPR / 64;      // chunks of a tile per lane
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 15, lg = lane >> 4;
-  const int xor16 = 4 * (lane ^ 16), xor32 = 4 * (lane ^ 32);
   const int seq = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int G = Hq / Hkv;
   const int head0 = kvh * G;
@@ -636,8 +635,8 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
         st[u][i] = sc;
         tmax = fmaxf(tmax, sc);
       }
-    tmax = fmaxf(tmax, __int_as_float(__builtin_amdgcn_ds_bpermute(xor16, __float_as_int(tmax))));
-    tmax = fmaxf(tmax, __int_as_float(__builtin_amdgcn_ds_bpermute(xor32, __float_as_int(tmax))));
+    tmax = max_with_lane_xor16(tmax);
+    tmax = max_with_lane_xor32(tmax);
     if (tmax > m_run) {                                 // (finite: key kc is in range)
       const float alpha = __builtin_amdgcn_exp2f(m_run - tmax);
       m_run = tmax;

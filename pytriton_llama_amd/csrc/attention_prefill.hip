@@ -43,10 +43,6 @@
 // assembly for it: the compiler inserts the wait states between an MFMA and the first read of
 // its result only for instructions it knows.)
 __device__ __forceinline__ float max2(float a, float b) { return fmaxf(a, b); }
-// the value of lane (lane ^ k); addr = 4 * (lane ^ k)
-__device__ __forceinline__ float lane_xor(float x, int addr) {
-  return __int_as_float(__builtin_amdgcn_ds_bpermute(addr, __float_as_int(x)));
-}
 __device__ __forceinline__ s16x4_t lds_read_tr16(const bf16_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)p);
 }
@@ -78,7 +74,6 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 15, lg = lane >> 4;
-  const int xor16 = 4 * (lane ^ 16), xor32 = 4 * (lane ^ 32);
   // Heads run along x, the fast index of the launch, so that workgroups started one after the
   // other land on the eight XCDs in turn; the heads are dealt out so that XCD c gets heads
   // c * Hq/8 .. (c+1) * Hq/8 - 1: the query heads of a kv head meet in one L2, which then holds
@@ -266,8 +261,8 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t
       for (int kt = 0; kt < 4; ++kt)
         tm[kt] = max2(max2(st[r][kt][0], st[r][kt][1]), max2(st[r][kt][2], st[r][kt][3]));
       float tmax = max2(max2(tm[0], tm[1]), max2(tm[2], tm[3]));
-      tmax = max2(tmax, lane_xor(tmax, xor16));
-      tmax = max2(tmax, lane_xor(tmax, xor32));
+      tmax = max_with_lane_xor16(tmax);
+      tmax = max_with_lane_xor32(tmax);
       // the maximum moved far enough for this lane's row: rescale what is kept. (A branch per
       // lane, not per wave: the lanes that skip it keep their registers, so nothing is copied
       // where it joins.)

@@ -18,3 +18,17 @@ union Frag8 {
   s16x4_t s[2];
   bf16x8_t v;
 };
+
+// The larger of x in this lane and in lane ^ 16 (lane ^ 32): gfx950 swaps the odd rows of 16 (32)
+// lanes of one register with the even rows of another in one VALU instruction; with both
+// registers holding x, one then holds the even rows' values everywhere and the other the odd
+// rows'. A ds_bpermute for the same costs a trip through the LDS crossbar, some hundred cycles
+// in the chain of every key tile.
+__device__ __forceinline__ float max_with_lane_xor16(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_with_lane_xor32(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
