@@ -127,11 +127,51 @@ def test_llama3_bands_of_tiny_b():
     torch.testing.assert_close(got[kept], base[kept])
     torch.testing.assert_close(got[divided], base[divided] / 8)
     assert torch.all(got[mid] > base[mid] / 8) and torch.all(got[mid] < base[mid])
-    # the blend meets both bands at their edges
-    for wl, want in ((64 / 4, 1.0), (64 / 1, 1 / 8)):
-        inv = torch.tensor([2 * math.pi / wl])
-        smooth = (64 / wl - 1.0) / (4.0 - 1.0)
-        assert abs(((1 - smooth) / 8 + smooth) - want) < 1e-12
+
+
+def _both_llama3(theta, dim, sc):
+    """The plain function and the product's, on the same numbers."""
+    from pytriton_llama_amd.parts.rotary import llama3_inv_freq
+    return (pl.rope_inv_freq_llama3(theta, dim, sc),
+            llama3_inv_freq(theta, dim, sc["factor"], sc["low_freq_factor"], sc["high_freq_factor"],
+                            sc["original_max_position_embeddings"]))
+
+
+@pytest.mark.parametrize("at, weight_of_kept", [(0.0, 0.0), (0.25, 0.25), (0.5, 0.5), (0.9, 0.9), (1.0, 1.0)])
+def test_llama3_blend_weight_at_constructed_wavelengths(at, weight_of_kept):
+    # RotaryEmbedding.py:90-98. dim 4 has the frequencies 1 and theta^-1/2; the original length
+    # is chosen so that original / wavelength of the second lies at low + at * (high - low):
+    # at = 0 is the edge of the divided band (result inv / factor), at = 1 the edge of the kept
+    # band (result inv), and between them the kept share grows linearly with ``at``. A blend
+    # weight the wrong way round (smooth <-> 1 - smooth) gives 0.75 where 0.25 is due.
+    theta, factor, low, high = 400.0, 8.0, 1.0, 4.0
+    inv = 1.0 / math.sqrt(theta)
+    wavelen = 2 * math.pi / inv
+    original = (low + at * (high - low)) * wavelen
+    sc = {"factor": factor, "low_freq_factor": low, "high_freq_factor": high,
+          "original_max_position_embeddings": original}
+    want = inv * (weight_of_kept + (1.0 - weight_of_kept) / factor)
+    for got in _both_llama3(theta, 4, sc):
+        assert got.dtype == torch.float32 and got.shape == (2,)
+        assert float(got[0]) == 1.0                                   # wavelength 2 pi: kept
+        assert abs(float(got[1]) - want) <= 2e-6 * want, (float(got[1]), want)
+
+
+def test_llama3_values_of_the_1b_parameters():
+    # theta 5e5, head size 64, factor 32, low 1, high 4, original 8192 (Llama-3.2-1B's
+    # config.json). Worked out in float64 outside both implementations: wavelengths below 2,048
+    # are kept (j <= 14), above 8,192 divided by 32 (j >= 18), and j = 15, 16, 17 lie between
+    # (2,948.30, 4,442.88 and 6,695.11): 8192 / wavelength = 2.7785, 1.8438, 1.2236, so the kept
+    # share is 0.5928, 0.2813 and 0.0745.
+    sc = {"factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+          "original_max_position_embeddings": 8192}
+    want = {0: 1.0, 13: 0.004839421345719893, 14: 0.003211445994752591,
+            15: 0.0012905479282092638, 16: 0.0004295567965593682, 17: 9.70828780262767e-05,
+            18: 1.9461638184831125e-05, 19: 1.291476718704739e-05, 31: 9.41830672543491e-08}
+    for got in _both_llama3(5e5, 64, sc):
+        assert got.shape == (32,)
+        for j, w in want.items():
+            assert abs(float(got[j]) - w) <= 3e-6 * w, (j, float(got[j]), w)
 
 
 def test_rope_parameters_of_the_reference_unit_test():
