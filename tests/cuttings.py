@@ -85,3 +85,54 @@ def max_live_tokens(steps, round_to=64):
         for rid in st["end"]:
             held.pop(rid, None)
     return peak
+
+
+def decoders_beside_a_portion(shorts, long_id, long_tokens, tails, portion=24, per_step=8,
+                              want_prompt_rows="all"):
+    """Many requests that decode together beside one prompt that arrives in portions.
+
+    ``shorts``: {request: tokens}; request r decodes its last ``tails[r]`` tokens one by one
+    (the others before them go in as one entry, ``per_step`` requests a step). Then every step
+    brings one token of every short request that still has some, and a portion of ``long_id``
+    while it lasts; with different tails the number of decoding rows falls from step to step.
+    ``want_prompt_rows``: "all" rows of the prompt entries or only their "last"."""
+    def prompt_entry(rid, toks, lo, hi):
+        e = _entry(rid, toks, lo, hi)
+        if want_prompt_rows == "last":
+            e["want"] = [hi - lo - 1]
+        return e
+
+    steps = []
+    ids = list(shorts)
+    for i in range(0, len(ids), per_step):
+        steps.append({"step": len(steps), "end": [], "entries": [
+            prompt_entry(r, shorts[r], 0, len(shorts[r]) - tails[r]) for r in ids[i:i + per_step]]})
+    done_long, s = 0, 0
+    while done_long < len(long_tokens) or any(s < tails[r] for r in ids):
+        entries, ended = [], []
+        for r in ids:
+            if s < tails[r]:
+                at = len(shorts[r]) - tails[r] + s
+                entries.append(_entry(r, shorts[r], at, at + 1))
+                if s == tails[r] - 1:
+                    ended.append(r)
+        if done_long < len(long_tokens):
+            hi = min(len(long_tokens), done_long + portion)
+            entries.append(prompt_entry(long_id, long_tokens, done_long, hi))
+            done_long = hi
+            if hi == len(long_tokens):
+                ended.append(long_id)
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+        s += 1
+    return steps
+
+
+def wanted_places(steps):
+    """{request: sorted positions whose logits the steps ask for}."""
+    fed, out = {}, {}
+    for st in steps:
+        for e in st["entries"]:
+            base = fed.get(e["id"], 0)
+            out.setdefault(e["id"], []).extend(base + w for w in e["want"])
+            fed[e["id"]] = base + len(e["tokens"])
+    return {r: sorted(p) for r, p in out.items()}
