@@ -17,7 +17,9 @@
 // probability are kept or dropped together; a sort would split such a tie at
 // the edge of the nucleus by index.
 #include "common.h"
+#include "no_alloc.h"
 #include <math.h>
+#include <mutex>
 
 // Two passes so that a row of vocabulary size is read by many workgroups: every
 // chunk leaves its best (value, index), then one wave per row picks among them.
@@ -97,6 +99,47 @@ extern "C" int ptl_argmax(int32_t* out, const float* logits, int R, int V, long 
   if (hipGetLastError() != hipSuccess) return PTL_ERR_LAUNCH;
   argmax_final_kernel<<<R, 64, 0, stream>>>(out, ws_val, ws_idx, chunks, host_out);
   return ptl_launch_status();
+}
+
+// ptl_argmax with its workspace inside the library (see no_alloc.h): values in the first half of
+// the array, indices in the second. Host code never uses the array's name as an address: the
+// name is a host-side stand-in; the device address comes from hipGetSymbolAddress, once per
+// device with that device current (every GPU holds a copy of its own), and is what the
+// kernels are given.
+static __device__ __align__(256) unsigned char argmax_scratch[PTL_ARGMAX_STATIC_MAX_PARTIALS * 8];
+#define ARGMAX_STATIC_MAX_DEVICES 64
+static void* argmax_scratch_at[ARGMAX_STATIC_MAX_DEVICES];
+static std::mutex argmax_scratch_lock;
+
+static int argmax_scratch_of_current_device(void** base) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ARGMAX_STATIC_MAX_DEVICES) return PTL_ERR_LAUNCH;
+  std::lock_guard<std::mutex> hold(argmax_scratch_lock);
+  if (argmax_scratch_at[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return PTL_ERR_LAUNCH;
+    }
+    argmax_scratch_at[dev] = p;
+  }
+  *base = argmax_scratch_at[dev];
+  return PTL_OK;
+}
+
+extern "C" int ptl_argmax_static(int32_t* out, const float* logits, int R, int V, long stride,
+                                 int32_t* host_out, hipStream_t stream) {
+  if (R <= 0) return PTL_OK;
+  if (!out || !logits || V <= 0 || stride < V || R > 65535) return PTL_ERR_ARG;
+  const long chunks = ((long)V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+  if ((long)R * chunks > PTL_ARGMAX_STATIC_MAX_PARTIALS) return PTL_ERR_ARG;
+  void* base = nullptr;
+  const int rc = argmax_scratch_of_current_device(&base);
+  if (rc != PTL_OK) return rc;
+  float* ws_val = reinterpret_cast<float*>(base);
+  int32_t* ws_idx = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(base) +
+                                               (size_t)PTL_ARGMAX_STATIC_MAX_PARTIALS * 4);
+  return ptl_argmax(out, logits, R, V, stride, ws_val, ws_idx, host_out, stream);
 }
 
 // probs_out (optional, [R, V]) receives the renormalised nucleus distribution.
