@@ -12,7 +12,9 @@ host-side bookkeeping: no device call, no synchronisation.
 Cache layers with the same needs form a group; a group has a page pool and, for
 every live request, a block table of its own. Beside the pages every live
 request owns one state slot 0..max_num_seqs-1: the row of the device block
-tables and of every fixed-size state tensor that belongs to it.
+tables and of every fixed-size state tensor that belongs to it. One more slot,
+``padding_slot`` = max_num_seqs, belongs to nobody: rows that pad a step to the size of a
+recorded graph name it, so that a mixer with state reads and writes there and harms no request.
 """
 from __future__ import annotations
 
@@ -126,6 +128,7 @@ class CacheManager:
         for g, n in zip(self.paged, num_pages):
             g.pool = PagePool(n)
         self._free_slots: List[int] = list(range(self.max_num_seqs - 1, -1, -1))
+        self.padding_slot = self.max_num_seqs        # the state row of rows that pad a step
         self.slot_of: Dict[Hashable, int] = {}
         self.num_tokens: Dict[Hashable, int] = {}
 

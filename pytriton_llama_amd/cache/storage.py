@@ -23,7 +23,8 @@ class PagedLayerView:
 @dataclass
 class StateLayerView:
     """What a mixer sees of one fixed-size-state cache layer."""
-    state: torch.Tensor        # [max_num_seqs, *shape], row = the request's state slot
+    state: torch.Tensor        # [max_num_seqs + 1, *shape], row = the request's state slot; the
+                               # last row is the padding slot (rows that pad a replayed step)
     group: int
     writable: bool
     kind: str = "state"
@@ -33,7 +34,8 @@ class CacheStorage:
     """Page pools [layers, num_pages, Hkv, page_size, D] for keys and for values
     per paged group (the reference keeps one [max_tokens, 2*Hkv, D] tensor per
     layer, lite_llama/executor/mem_manager.py:166-168), and one
-    [layers, max_num_seqs, *shape] tensor per state group."""
+    [layers, max_num_seqs + 1, *shape] tensor per state group (the last row is the padding
+    slot of the manager)."""
 
     def __init__(self, manager: CacheManager, dtype: torch.dtype, device):
         self.manager = manager
@@ -46,7 +48,7 @@ class CacheStorage:
             self.k_pools.append(torch.zeros(shape, dtype=dtype, device=device))
             self.v_pools.append(torch.zeros(shape, dtype=dtype, device=device))
         for g in manager.states:
-            shape = (len(g.layers), manager.max_num_seqs) + tuple(g.spec.shape)
+            shape = (len(g.layers), manager.max_num_seqs + 1) + tuple(g.spec.shape)
             self.state_pools.append(torch.zeros(shape, dtype=g.spec.dtype or dtype, device=device))
 
     def view(self, cache_layer: Optional[int], writable: bool = True):
@@ -65,6 +67,19 @@ class CacheStorage:
         """A new request starts from zero state."""
         for pool in self.state_pools:
             pool[:, slot].zero_()
+
+    @staticmethod
+    def state_bytes(manager: CacheManager, dtype: torch.dtype) -> int:
+        """Bytes of the fixed-size state of all slots (what the state pools take whatever the
+        number of pages)."""
+        total = 0
+        for g in manager.states:
+            size = torch.empty((), dtype=g.spec.dtype or dtype).element_size()
+            n = 1
+            for d in g.spec.shape:
+                n *= int(d)
+            total += len(g.layers) * (manager.max_num_seqs + 1) * n * size
+        return total
 
     @staticmethod
     def bytes_per_page(manager: CacheManager, dtype: torch.dtype) -> int:

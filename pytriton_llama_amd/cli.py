@@ -1,6 +1,7 @@
 """Command line in the reference's manner (cli.py:11-66): the same option names
 with the same meanings (temperature, top_p, max_seq_len, max_gpu_num_blocks,
-max_gen_len, load_model, compiled_model, triton_weight), the checkpoint folder
+max_gen_len, load_model, compiled_model, triton_weight; compiled_model is on
+unless switched off, because the replayed step is the fast path here), the checkpoint folder
 as an option instead of a line to edit in the source, and a prompt loop that
 ends at "exit". With a tokenizer.json in the folder prompts are text; without
 one they are token ids separated by blanks or commas.
@@ -28,7 +29,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max_gpu_num_blocks", type=int, default=None, help="cache pages (None: from free memory)")
     ap.add_argument("--max_gen_len", type=int, default=1024)
     ap.add_argument("--load_model", type=_bool, default=True, help="false: random weights from --seed")
-    ap.add_argument("--compiled_model", type=_bool, default=False, help="replay decode steps as HIP graphs")
+    ap.add_argument("--compiled_model", type=_bool, default=True,
+                    help="replay decode steps and single prompt portions as HIP graphs (false: launch "
+                         "every kernel from the host)")
     ap.add_argument("--triton_weight", type=_bool, default=True, help="accepted, without effect")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--seed", type=int, default=0)

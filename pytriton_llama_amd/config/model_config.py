@@ -69,6 +69,7 @@ class LlamaConfig:
     rope_theta: float
     rope_scaling: RopeScaling
     tie_word_embeddings: bool
+    tie_word_embeddings_given: bool = True    # False: config.json has no such key (tied by default)
     max_position_embeddings: Optional[int] = None
     bos_token_id: Optional[int] = None
     eos_token_id: Any = None
@@ -138,7 +139,11 @@ class LlamaConfig:
             rms_norm_eps=float(d.get("rms_norm_eps", 1e-5)),
             rope_theta=float(d.get("rope_theta", 10000.0)),
             rope_scaling=RopeScaling.from_dict(d.get("rope_scaling")),
+            # absent: tied, as the reference's LlamaConfig has it
+            # (lite_llama/models/model_config.py:37-104); a checkpoint that then brings a head of
+            # its own is refused by the loader rather than run with the embedding table
             tie_word_embeddings=bool(d.get("tie_word_embeddings", True)),
+            tie_word_embeddings_given=d.get("tie_word_embeddings") is not None,
             max_position_embeddings=d.get("max_position_embeddings"),
             bos_token_id=d.get("bos_token_id"),
             eos_token_id=d.get("eos_token_id"),
@@ -181,6 +186,8 @@ class LlamaConfig:
                     "original_max_position_embeddings": v.original_max_position_embeddings}
             elif isinstance(v, tuple):
                 v = list(v)
+            if f.name == "tie_word_embeddings_given":
+                continue
             d[f.name] = v
         d["hidden_act"] = "silu"
         d["attention_bias"] = False

@@ -28,6 +28,34 @@ __global__ void add_rmsnorm_kernel(T* __restrict__ y, const T* __restrict__ x,
     y[base + i] = from_float<T>(row[i] * rr * w[i]);
 }
 
+// Rows too wide for the LDS copy above: two passes over memory. The first adds up the squares of
+// the sums without storing them, the second makes the sums again (from the same inputs, so they
+// are the same numbers), stores them as the new residual and writes the result. Every element is
+// read and written by one thread only, so y may be x.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+add_rmsnorm_wide_kernel(T* __restrict__ y, const T* __restrict__ x, T* __restrict__ residual,
+                        const float* __restrict__ w, int H, float eps, int has_residual) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = to_float<T>(x[base + i]);
+    if (has_residual) v += to_float<T>(residual[base + i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float rr = 1.0f / sqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = to_float<T>(x[base + i]);
+    if (has_residual) {
+      v += to_float<T>(residual[base + i]);
+      residual[base + i] = from_float<T>(v);
+    }
+    y[base + i] = from_float<T>(v * rr * w[i]);
+  }
+}
+
 // bfloat16 rows whose width is a multiple of 8: 16-byte loads, the summed row stays in
 // registers (CH chunks of 8 elements per thread), one pass over memory.
 template <int CH>
@@ -80,7 +108,7 @@ add_rmsnorm_bf16_vec_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x
 extern "C" int ptl_add_rmsnorm(void* y, const void* x, void* residual, const float* w,
                                int T_, int H, float eps, int dtype, hipStream_t stream) {
   if (T_ <= 0) return PTL_OK;
-  if (H <= 0 || (size_t)H * 4 > 60000) return PTL_ERR_ARG;
+  if (H <= 0) return PTL_ERR_ARG;
   if (dtype == PTL_DTYPE_BF16 && H % 8 == 0 && H <= 8 * 256 * 4 &&
       ((uintptr_t)x | (uintptr_t)y | (uintptr_t)residual | (uintptr_t)w) % 16 == 0) {
     const int nchunk = H / 8;
@@ -98,6 +126,17 @@ extern "C" int ptl_add_rmsnorm(void* y, const void* x, void* residual, const flo
   while (threads < 1024 && threads * 4 < H) threads <<= 1;
   const size_t lds = (size_t)H * sizeof(float);
   const int has_res = residual != nullptr;
+  if (lds > 60000) {        // the row does not fit the LDS a workgroup may ask for
+    if (dtype == PTL_DTYPE_F32)
+      add_rmsnorm_wide_kernel<float><<<T_, 1024, 0, stream>>>(
+          (float*)y, (const float*)x, (float*)residual, w, H, eps, has_res);
+    else if (dtype == PTL_DTYPE_BF16)
+      add_rmsnorm_wide_kernel<bf16_t><<<T_, 1024, 0, stream>>>(
+          (bf16_t*)y, (const bf16_t*)x, (bf16_t*)residual, w, H, eps, has_res);
+    else
+      return PTL_ERR_ARG;
+    return ptl_launch_status();
+  }
   if (dtype == PTL_DTYPE_F32)
     add_rmsnorm_kernel<float, 1><<<T_, threads, lds, stream>>>(
         (float*)y, (const float*)x, (float*)residual, w, H, eps, has_res);

@@ -8,8 +8,9 @@ a step whose entries all bring one token runs through a graph captured once per
 batch-size bucket: the integer tables of the step live in one static device
 buffer that is refreshed by a single copy from pinned host memory, then the
 graph is replayed. Rows beyond the live sequences are padding: they have
-ctx_len 0 (attention reads nothing), slot -1 (nothing is written to the cache)
-and their logits are dropped.
+ctx_len 0 (attention reads nothing), cache slot -1 (nothing is written to the
+cache pages), the manager's padding slot as state slot (a mixer with state of its own
+reads and writes a row that belongs to no request) and their logits are dropped.
 
 A step with one entry of several tokens (a prompt, or a portion of one: the first thing a
 request sees on an engine that is idle or only decoding) is some 150 launches that cost the
@@ -19,7 +20,13 @@ every 128 up to 2,048) and
 of the number of single-token entries beside it (0, 1, 2, 4, ...):
 the tokens are padded to the bucket with rows that write nothing to the cache (slot -1) and
 that no query block covers (the work lists name blocks up to the bucket's size; a block
-past the real tokens is empty and its workgroup leaves at once).
+past the real tokens is empty and its workgroup leaves at once). The device tensors of the
+context (q_start above all) say where the real tokens end; the host copies in the context of
+a recorded step (q_lens, ctx_lens and the maxima) are the bucket's upper bounds. A mixer with
+state of its own must stop at q_start[i + 1], not at the padded length.
+
+All graphs of a runner share one memory pool: they are replayed one at a time on one stream,
+so what a step needs while it runs is the most that any of them needs, not the sum.
 
 Nothing in a captured step clears memory with a memset node, and the buffers a
 replay reads are written by ordinary copies before it.
@@ -101,8 +108,10 @@ class _Bucket:
         return self.np[a:a + k]
 
 
-def capture_forward(model, storage, ctx, device):
-    """(graph, logits) of one forward pass over ``ctx``, whose tensors are static buffers."""
+def capture_forward(model, storage, ctx, device, pool=None):
+    """(graph, logits) of one forward pass over ``ctx``, whose tensors are static buffers.
+    ``pool``: the memory pool the graph's tensors come from (shared by graphs that never run
+    at the same time)."""
     side = torch.cuda.Stream(device=device)
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -110,18 +119,16 @@ def capture_forward(model, storage, ctx, device):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    with torch.cuda.graph(graph, pool=pool):
         logits = model.forward(ctx, storage)
     return graph, logits
 
 
 class DecodeGraphs:
-    def __init__(self, model, manager, storage, max_model_len: int, device):
-        if manager.states:
-            raise ValueError("padding rows would touch state slots: models with fixed-size "
-                             "state do not run through decode graphs")
+    def __init__(self, model, manager, storage, max_model_len: int, device, pool=None):
         self.model, self.manager, self.storage = model, manager, storage
         self.device = device
+        self.pool = pool
         self.max_model_len = int(max_model_len)
         self.width = -(-self.max_model_len // manager.page_size)
         self.sizes = bucket_sizes(manager.max_num_seqs)
@@ -148,7 +155,7 @@ class DecodeGraphs:
         # the split of the decode attention is fixed at capture: plan it for the longest context
         b.ctx.ctx_lens = [self.max_model_len] * b.size
         b.ctx.max_ctx_len = self.max_model_len
-        b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device)
+        b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device, self.pool)
 
     def step(self, entries: Sequence[StepEntry], token_feed=None) -> torch.Tensor:
         """Logits [wanted, vocab] of a step whose entries all bring one token.
@@ -169,7 +176,9 @@ class DecodeGraphs:
         ctx[:n] = starts
         ctx[:n] += 1
         ctx[n:] = 0
-        np_("state_slots")[:n] = [m.slot_of[e.request] for e in entries]
+        slot_of = np_("state_slots")
+        slot_of[:n] = [m.slot_of[e.request] for e in entries]
+        slot_of[n:] = m.padding_slot
         P = m.page_size
         for g, group in enumerate(m.paged):
             slots = np_(f"slots{g}")
@@ -191,8 +200,14 @@ class DecodeGraphs:
             # tokens the step before left on the device
             ops.stage_step(b.dev, b.host, token_feed, b.spans["token_ids"][0], n)
         if b.graph is None:
+            # Recording runs the step once for real beforehand. Keys and values written twice
+            # are the same keys and values, but a mixer with state of its own would take the
+            # step twice: while recording, every row's state is the padding slot's.
+            real = slot_of.copy()
+            slot_of[:] = m.padding_slot
             refresh()
-            self._capture(b)
+            self._capture(b)                      # waits for the device at its end
+            slot_of[:] = real
             b.copied = torch.cuda.Event()
         refresh()
         b.copied.record()
@@ -281,12 +296,10 @@ class PortionGraphs:
     """Steps of single-token entries (any number up to the largest decode bucket, also none)
     and exactly one entry of 2 to 2,048 tokens with at most one wanted place."""
 
-    def __init__(self, model, manager, storage, max_model_len: int, device):
-        if manager.states:
-            raise ValueError("padding rows would touch state slots: models with fixed-size "
-                             "state do not run through graphs")
+    def __init__(self, model, manager, storage, max_model_len: int, device, pool=None):
         self.model, self.manager, self.storage = model, manager, storage
         self.device = device
+        self.pool = pool
         self.max_model_len = int(max_model_len)
         self.width = -(-self.max_model_len // manager.page_size)
         self.sizes = list(PORTION_BUCKETS)
@@ -359,7 +372,7 @@ class PortionGraphs:
         np_("q_start")[B + 1] = B + n
         slot_of = np_("state_slots")
         slot_of[:k] = [m.slot_of[entries[i].request] for i in ones]
-        slot_of[k:B] = 0
+        slot_of[k:B] = m.padding_slot
         slot_of[B] = m.slot_of[e.request]
         np_("logit_rows")[B] = B + (e.want[0] if e.want else n - 1)
         P = m.page_size
@@ -376,11 +389,16 @@ class PortionGraphs:
             table = group.tables[e.request]
             table_np[B, :len(table)] = table
             table_np[B, len(table):] = -1
-        b.dev.copy_(b.host, non_blocking=True)
         if b.graph is None:
-            b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device)
+            # (as for decode steps: no request's state is touched by the run that records)
+            real = slot_of.copy()
+            slot_of[:] = m.padding_slot
             b.dev.copy_(b.host, non_blocking=True)
+            b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device,
+                                                self.pool)
+            slot_of[:] = real
             b.copied = torch.cuda.Event()
+        b.dev.copy_(b.host, non_blocking=True)
         b.copied.record()
         b.graph.replay()
         # rows of the graph's logits in the caller's order of entries (a copy: the next replay

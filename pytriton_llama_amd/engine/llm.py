@@ -18,20 +18,34 @@ from .runner import ModelRunner
 from .scheduler import Scheduler
 
 
+def pages_that_fit(usable_bytes: int, bytes_per_page: int, state_bytes: int, cap: int) -> int:
+    """Pages for ``usable_bytes`` of memory when the fixed-size state of all slots takes
+    ``state_bytes`` of it first; at most ``cap``. A model without paged layers needs no page
+    (one is kept so that the pools exist)."""
+    left = usable_bytes - state_bytes
+    if left < 0:
+        raise RuntimeError(f"the fixed-size state of the requests ({state_bytes} bytes) does not fit "
+                           f"into the {max(usable_bytes, 0)} bytes left after loading the weights")
+    if bytes_per_page <= 0:
+        return 1
+    n = min(left // bytes_per_page, cap)
+    if n < 1:
+        raise RuntimeError("no memory left for the cache after loading the weights")
+    return int(n)
+
+
 def pages_from_memory(model, engine: EngineConfig) -> int:
     """Pages that fit into gpu_memory_fraction of the device after the weights
     are loaded (the reference: (total*0.9 - peak - non_torch) // bytes per block,
-    lite_llama/executor/mem_manager.py:44-60,98-110)."""
+    lite_llama/executor/mem_manager.py:44-60,98-110), less what the state pools take."""
     probe = CacheManager(model.cache_layers, engine.page_size, 1, engine.max_num_seqs)
     per_page = CacheStorage.bytes_per_page(probe, engine.dtype)
+    fixed = CacheStorage.state_bytes(probe, engine.dtype)
     free, total = torch.cuda.mem_get_info(torch.device(engine.device))
     usable = int(total * engine.gpu_memory_fraction) - (total - free)
     # no request can use more than max_model_len, and max_num_seqs of them may live
     cap = engine.max_num_seqs * (-(-engine.max_model_len // engine.page_size))
-    n = min(max(usable // max(per_page, 1), 0), cap)
-    if n < 1:
-        raise RuntimeError("no memory left for the cache after loading the weights")
-    return n
+    return pages_that_fit(usable, per_page, fixed, cap)
 
 
 class _Launched:

@@ -33,11 +33,14 @@ class ModelRunner:
         # decode-only steps replay a HIP graph when the longest request is known
         self.graphs = None
         self.portion_graphs = None
-        if use_graphs and max_model_len and self.device.type == "cuda" and not self.manager.states:
+        if (use_graphs and max_model_len and self.device.type == "cuda"
+                and model.graph_capturable()):
             from .graphs import DecodeGraphs, PortionGraphs
-            self.graphs = DecodeGraphs(model, self.manager, self.storage, max_model_len, self.device)
+            pool = torch.cuda.graph_pool_handle()
+            self.graphs = DecodeGraphs(model, self.manager, self.storage, max_model_len, self.device,
+                                       pool)
             self.portion_graphs = PortionGraphs(model, self.manager, self.storage, max_model_len,
-                                                self.device)
+                                                self.device, pool)
 
     def admit(self, request: Hashable) -> None:
         slot = self.manager.admit(request)

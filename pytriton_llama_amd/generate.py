@@ -36,13 +36,17 @@ class GenerateText:
     """checkpoints_dir: model folder (config.json + safetensors). max_seq_len
     caps prompt + generated tokens. max_gpu_num_blocks: size of the cache pool in
     pages (None: from free memory). load_model False starts from random weights
-    (seeded) instead of reading the folder's tensors. triton_weight and
-    compiled_model are accepted for compatibility: there is one weight format,
-    and compiled_model switches HIP-graph replay of decode steps."""
+    (seeded) instead of reading the folder's tensors. triton_weight is accepted
+    for compatibility (there is one weight format). compiled_model switches the
+    replay of decode steps and of single prompt portions as HIP graphs, and with
+    it the launch of a decode step ahead of the tokens of the step before; it is
+    on by default (the reference's flag defaults to off, lite_llama/generate.py:59,
+    and its captured graphs are never replayed, model_executor.py:314-320; here
+    the replayed step is the fast path and the one that is measured)."""
 
     def __init__(self, checkpoints_dir: str, tokenizer_path: Optional[str] = None,
                  max_seq_len: int = 1024, max_gpu_num_blocks: Optional[int] = None,
-                 load_model: bool = True, triton_weight: bool = True, compiled_model: bool = False,
+                 load_model: bool = True, triton_weight: bool = True, compiled_model: bool = True,
                  device: str = "cuda", dtype: str = "bfloat16", seed: int = 0,
                  page_size: int = 16, max_batch_size: int = 64,
                  max_num_batched_tokens: int = 2048, prefill_chunk: Optional[int] = None):

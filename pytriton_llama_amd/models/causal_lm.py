@@ -68,6 +68,11 @@ class CausalLM:
             libs += tuple(part.kernel_libraries)
         return tuple(dict.fromkeys(libs))
 
+    def graph_capturable(self) -> bool:
+        """Whether a step of this model can be recorded as a HIP graph: every part says so."""
+        return all(getattr(p, "graph_capturable", True)
+                   for p in [self.embedding, *self.blocks, self.final_norm, self.head])
+
     @property
     def vocab_size(self) -> int:
         return self.head.vocab_size
@@ -85,7 +90,7 @@ class CausalLM:
             # take it (parts/base.py); the rows for the final norm are picked first, so not there
             after = self.blocks[self.schedule[i + 1].block] if i < last else None
             if (after is not None and getattr(block, "can_defer_output", False)
-                    and getattr(getattr(after, "input_norm", None), "takes_pending_product", False)):
+                    and getattr(after, "takes_pending_product", False)):
                 h, residual = block.forward(h, residual, ctx, cache, defer_output=True)
             else:
                 h, residual = block.forward(h, residual, ctx, cache)

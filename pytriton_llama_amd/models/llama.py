@@ -74,8 +74,11 @@ def build_llama(cfg: LlamaConfig) -> CausalLM:
             prefixes.append((f"model.layers.{i}.{LLAMA_BLOCK_PREFIXES[role]}", part))
     prefixes += [("model.norm.", final_norm), ("lm_head.", head)]
     ignorable = ["*.rotary_emb.inv_freq"]
-    if cfg.tie_word_embeddings:
-        ignorable.append("lm_head.weight")      # a tied checkpoint may still carry the copy
+    if cfg.tie_word_embeddings and cfg.tie_word_embeddings_given:
+        # a checkpoint that says it is tied may still carry the copy. Without the key the model
+        # is tied by default, and a head in the file then means the default is wrong for it: it
+        # is reported as unexpected instead of being dropped silently
+        ignorable.append("lm_head.weight")
     cache_layers = [b.cache_spec() for b in blocks]
     schedule = [LayerCall(i, i) for i in range(len(blocks))]
     return CausalLM(cfg, embedding, blocks, final_norm, head, cache_layers, schedule, prefixes,

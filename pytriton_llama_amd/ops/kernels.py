@@ -119,8 +119,6 @@ def add_rmsnorm(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch
     if residual is not None and (residual.shape != x.shape or residual.dtype != x.dtype
                                  or not residual.is_contiguous()):
         raise KernelError("add_rmsnorm: residual must match x in shape and dtype")
-    if H * 4 > 60000:
-        raise KernelError(f"add_rmsnorm: width {H} exceeds the kernel's limit of 15000")
     y = out if out is not None else torch.empty_like(x)
     lib = library.load("norm")
     _check(lib.ptl_add_rmsnorm(_ptr(y), _ptr(x), _ptr(residual), _ptr(weight), T, H,
@@ -553,6 +551,12 @@ def _compute_units(device_index: int) -> int:
     return int(torch.cuda.get_device_properties(device_index).multi_processor_count)
 
 
+def compute_units(device) -> int:
+    """Compute units of the GPU ``device`` (256 on MI355X)."""
+    device = torch.device(device)
+    return _compute_units(device.index if device.index is not None else torch.cuda.current_device())
+
+
 def attention_prefill_mfma_plan(device: torch.device, num_heads: int, head_dim: int,
                                 blocks_of_64: int, blocks_of_128: int):
     """(block_rows, groups) for ``attention_prefill_mfma``, from sweeps on MI355X (one sequence
@@ -562,8 +566,7 @@ def attention_prefill_mfma_plan(device: torch.device, num_heads: int, head_dim: 
     before; a workgroup for every block while there are at most 2 t blocks (the longest start
     first and the short ones fill in behind them), beyond that t workgroups that share the
     sorted list as a snake, which evens out the causal triangle."""
-    index = device.index if device.index is not None else torch.cuda.current_device()
-    resident = _compute_units(index) * (3 if head_dim <= 64 else 2)
+    resident = compute_units(device) * (3 if head_dim <= 64 else 2)
     t = max(1, resident // num_heads)
     rows, blocks = (128, blocks_of_128) if 4 * blocks_of_128 >= 5 * t else (64, blocks_of_64)
     return rows, max(1, blocks if blocks <= 2 * t else t)

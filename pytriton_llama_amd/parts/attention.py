@@ -55,6 +55,10 @@ class PagedAttention(Part):
     def cache_spec(self):
         return PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
 
+    @property
+    def graph_capturable(self) -> bool:
+        return self.position is None or getattr(self.position, "graph_capturable", True)
+
     def param_sources(self) -> List[ParamSource]:
         qn, kn, vn, on = self.names
         return [ParamSource(qn, (self.q_size, self.hidden_size)),
@@ -110,9 +114,9 @@ class PagedAttention(Part):
         return linear(out.view(T, Hq * D), self.o)
 
     # ---- which kernel takes which sequences --------------------------------------
-    def decode_splits(self, ctx, n_dec: int, matrix_cores: bool) -> int:
-        """How many workgroups share one sequence's keys: enough to fill the 256
-        CUs a few times over, never finer than one turn of a workgroup."""
+    def decode_splits(self, ctx, n_dec: int, matrix_cores: bool, device) -> int:
+        """How many workgroups share one sequence's keys: enough to fill the compute
+        units a few times over, never finer than one turn of a workgroup."""
         if self.force_decode_splits:
             return self.force_decode_splits
         D = self.head_dim
@@ -129,14 +133,15 @@ class PagedAttention(Part):
         span = max(ctx.ctx_lens[:n_dec])
         if self.window:
             span = min(span, self.window)
-        # measured on MI355X: the matrix-core kernel is best with about 512 workgroups (one
-        # round over the 256 CUs) and without splits once the batch brings half of that; the
-        # other one with about a thousand
+        # measured on MI355X (256 compute units): the matrix-core kernel is best with about two
+        # workgroups a compute unit and without splits once the batch brings one for each; the
+        # other one with about four
         base = max(1, n_dec * groups)
+        cus = ops.compute_units(device)
         if matrix_cores:
-            want = 1 if base >= 256 else -(-512 // base)
+            want = 1 if base >= cus else -(-2 * cus // base)
         else:
-            want = -(-1024 // base)
+            want = -(-4 * cus // base)
         return max(1, min(want, -(-span // turn), 64))
 
     def attend(self, out, q, cache, ctx, group) -> None:
@@ -148,7 +153,7 @@ class PagedAttention(Part):
                     and q.stride(0) % 8 == 0)
             ops.attention_decode(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
                                  group.block_table, n_dec, self.scale, window,
-                                 self.decode_splits(ctx, n_dec, mfma), matrix_cores=mfma)
+                                 self.decode_splits(ctx, n_dec, mfma, q.device), matrix_cores=mfma)
         if n_dec == ctx.num_seqs:
             return
         if (ops.attention_prefill_mfma_fits(q.dtype, self.num_kv_heads, D, cache.page_size)

@@ -21,7 +21,9 @@ feed-forward:    forward(x) -> y
 position:        rotary_inv_freq() -> float32 [D/2] or None;  apply(q, k, positions) in place
 embedding:       forward(token_ids int32 [T]) -> [T, hidden]
 head:            forward(x [R, hidden]) -> float32 logits [R, vocab]
-block:           forward(h, residual, ctx, cache) -> (h, residual)
+block:           forward(h, residual, ctx, cache) -> (h, residual); may set the flags
+                 can_defer_output (forward then takes defer_output=True and may return a
+                 pending h) and takes_pending_product (its h may arrive pending)
 
 Work handed on instead of done (optional; a part that knows nothing of it is given tensors)
 ------------------------------------------------------------------------------------------
@@ -60,6 +62,10 @@ class ParamSource:
     shape: Tuple[int, ...]
     kind: str = "matrix"      # "matrix": held in the engine dtype; "vector": held in float32;
                               # "table": integers, held as int32
+    init: Optional[Tuple] = None   # how the random-weights mode draws it. None: by kind (matrix
+                              # N(0, std), vector 1 + N(0, norm_std): a norm weight, table
+                              # uniform integers). Else ("normal", mean, std), ("uniform", low,
+                              # high) or ("constant", value): biases, decay rates, gates
 
 
 @dataclass(frozen=True)
@@ -125,9 +131,12 @@ def run_norm(norm, x, residual, consumer=None):
 
 class Part:
     kernel_libraries: Tuple[str, ...] = ()
-    takes_pending_product = False     # norms
+    takes_pending_product = False     # norms, blocks
     takes_pending_scale = False       # mixers, feed-forwards
     can_defer_output = False          # mixers, feed-forwards, blocks
+    graph_capturable = True           # False: forward waits for the device or reads device data
+                                      # on the host; steps of a model with such a part are
+                                      # launched kernel by kernel, never replayed as graphs
 
     def param_sources(self) -> List[ParamSource]:
         return []

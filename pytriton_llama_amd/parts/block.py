@@ -29,6 +29,16 @@ class PreNormBlock(Part):
 
     can_defer_output = True
 
+    @property
+    def takes_pending_product(self) -> bool:
+        """Whether the block before this one may leave its last product to this block's first
+        norm (parts/base.py): what the model asks when it runs two blocks in a row."""
+        return bool(getattr(self.input_norm, "takes_pending_product", False))
+
+    @property
+    def graph_capturable(self) -> bool:
+        return all(getattr(p, "graph_capturable", True) for p in self.children().values())
+
     def forward(self, h, residual, ctx, cache, defer_output: bool = False):
         """``h`` may be pending work of the block before (parts/base.py); with ``defer_output``
         the feed-forward may leave its last product to whoever normalises next."""

@@ -4,7 +4,8 @@ The reference has no such mode (its only random tensor is a placeholder,
 lite_llama/models/llama.py:23). Every tensor is drawn in float32 on the host
 from a generator seeded by (seed, tensor name), so the values depend neither on
 the order of creation nor on the device nor on the dtype they are stored in:
-matrices ~ N(0, initializer_range), norm vectors 1 + N(0, norm_std).
+matrices ~ N(0, initializer_range), norm vectors 1 + N(0, norm_std), unless the part
+that owns a tensor says otherwise (ParamSource.init).
 """
 from __future__ import annotations
 
@@ -26,8 +27,22 @@ def _generator(seed: int, name: str) -> torch.Generator:
 
 
 def random_tensor(seed: int, name: str, shape, kind: str, std: float, norm_std: float,
-                  vocab: int = 0) -> torch.Tensor:
+                  vocab: int = 0, init=None) -> torch.Tensor:
+    """``init``: the part's own wish for this tensor (ParamSource.init), which goes before the
+    rule of its kind."""
     g = _generator(seed, name)
+    if init is not None:
+        how, *numbers = init
+        if how == "normal" and len(numbers) == 2:
+            t = numbers[0] + numbers[1] * torch.randn(shape, generator=g, dtype=torch.float32)
+        elif how == "uniform" and len(numbers) == 2:
+            t = numbers[0] + (numbers[1] - numbers[0]) * torch.rand(shape, generator=g, dtype=torch.float32)
+        elif how == "constant" and len(numbers) == 1:
+            t = torch.full(shape, float(numbers[0]), dtype=torch.float32)
+        else:
+            raise ValueError(f"tensor {name!r}: unknown init hint {init!r}; known: ('normal', mean, std), "
+                             "('uniform', low, high), ('constant', value)")
+        return t.round().to(torch.int32) if kind == "table" else t
     if kind == "vector":
         t = torch.ones(shape, dtype=torch.float32)
         if norm_std:
@@ -44,7 +59,8 @@ def random_tensors(model, seed: int, norm_std: float = 0.0,
     if std is None:
         std = float(getattr(model.config, "initializer_range", 0.02))
     for name, (part, src) in model.expected_tensors().items():
-        yield name, part, src, random_tensor(seed, name, src.shape, src.kind, std, norm_std)
+        yield name, part, src, random_tensor(seed, name, src.shape, src.kind, std, norm_std,
+                                             init=getattr(src, "init", None))
 
 
 def load_random_weights(model, seed: int, dtype: torch.dtype, device, norm_std: float = 0.0,

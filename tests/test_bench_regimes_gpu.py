@@ -194,3 +194,30 @@ def test_many_decoding_rows_at_real_widths(shape_folders, name, dtype, graphs):
     got = replay_wanted(runner, steps)
     bad = first_wrong_row(got, want, places, TOL[dtype])
     assert bad is None, f"shape {name}, {dtype}: first wrong place (request, position, error) = {bad}"
+
+
+@pytest.fixture(scope="module")
+def full_depth(tmp_path_factory, gpu_device):
+    """All sixteen layers of the 1B shape, as the measurements run it."""
+    from pytriton_llama_amd.weights import write_random_model
+    cfg = dict(SHAPES["1b"], num_hidden_layers=16)
+    folder = str(tmp_path_factory.mktemp("full_depth"))
+    write_random_model(cfg, folder, seed=6, dtype=torch.bfloat16, std=0.02)
+    seqs = random_sequences(cfg["vocab_size"], [260, 45, 150], seed=12)
+    steps = cuttings.mixed(seqs, seed=2, max_live=3)
+    for st in steps:                       # the last row of every entry is enough here
+        for e in st["entries"]:
+            e["want"] = e["want"][-1:]
+    places = cuttings.wanted_places(steps)
+    return folder, seqs, steps, places, plain_rows(folder, seqs, places)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_sixteen_layers_mixed(full_depth, dtype):
+    """The whole depth of the 1B shape (weights N(0, 0.02) as in the measurements): portions of
+    three prompts beside decoded tokens, against the plain model."""
+    folder, seqs, steps, places, want = full_depth
+    runner = load_runner(folder, dtype, 16, cuttings.max_live_tokens(steps) // 16, max_num_seqs=4)
+    got = replay_wanted(runner, steps)
+    bad = first_wrong_row(got, want, places, TOL[dtype])
+    assert bad is None, f"16 layers, {dtype}: first wrong place (request, position, error) = {bad}"

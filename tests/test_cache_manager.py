@@ -141,3 +141,27 @@ def test_random_orders_keep_the_books(seed):
         m.free(rid)
     m.check()
     assert all(g.pool.num_free == g.pool.num_pages for g in m.paged) and m.num_free_slots == 5
+
+
+def test_cache_sizing_counts_the_fixed_state():
+    """The state pools come out of the memory before the pages do."""
+    import torch
+    from pytriton_llama_amd.cache import CacheStorage
+    from pytriton_llama_amd.engine.llm import pages_that_fit
+    from pytriton_llama_amd.parts import PagedKVSpec, StateSpec
+    layers = [PagedKVSpec(2, 16), StateSpec((1000,), torch.float32), StateSpec((1000,), torch.float32),
+              PagedKVSpec(2, 16), StateSpec((8, 8), None)]
+    m = CacheManager(layers, 16, 4, 10)
+    assert m.padding_slot == 10 and m.padding_slot not in m._free_slots
+    per_page = CacheStorage.bytes_per_page(m, torch.bfloat16)
+    assert per_page == 2 * 2 * 2 * 16 * 16 * 2
+    fixed = CacheStorage.state_bytes(m, torch.bfloat16)
+    assert fixed == 2 * 11 * 1000 * 4 + 1 * 11 * 64 * 2          # every slot and the padding slot
+    assert pages_that_fit(fixed + 10 * per_page + 5, per_page, fixed, 1000) == 10
+    assert pages_that_fit(fixed + 10 * per_page + 5, per_page, 0, 1000) > 10
+    assert pages_that_fit(10 ** 9, per_page, fixed, 7) == 7
+    with pytest.raises(RuntimeError, match="fixed-size state"):
+        pages_that_fit(fixed - 1, per_page, fixed, 1000)
+    with pytest.raises(RuntimeError, match="no memory left"):
+        pages_that_fit(fixed + per_page - 1, per_page, fixed, 1000)
+    assert pages_that_fit(fixed, 0, fixed, 1000) == 1            # a model without paged layers

@@ -107,7 +107,8 @@ def test_seeded_temperature_sampling(folder_b):
     assert eng.generate(prompts[1:2], params[1:2])[0] == a[1]
 
 
-def test_command_line(folder_a):
+@pytest.mark.parametrize("compiled", ["true", "false"])
+def test_command_line(folder_a, compiled):
     folder, page = folder_a
     cfg, w = plain_llama.read_model_folder(folder)
     prompt = [7, 1, 30, 200, 11]
@@ -115,10 +116,109 @@ def test_command_line(folder_a):
     out = subprocess.run(
         [sys.executable, os.path.join(ROOT, "cli.py"), "--checkpoints_dir", folder, "--dtype", "float32",
          "--temperature", "0", "--max_gen_len", "5", "--max_seq_len", "64", "--max_gpu_num_blocks", "32",
-         "--page_size", str(page), "--prompt_ids", ",".join(map(str, prompt))],
+         "--page_size", str(page), "--compiled_model", compiled,
+         "--prompt_ids", ",".join(map(str, prompt))],
         capture_output=True, text=True, timeout=110)
     assert out.returncode == 0, out.stderr[-2000:]
     assert [int(x) for x in out.stdout.split()] == want
+
+
+def test_entry_points_replay_graphs_unless_told_otherwise(folder_a):
+    from pytriton_llama_amd.cli import build_parser
+    from pytriton_llama_amd.generate import GenerateText
+    folder, page = folder_a
+    assert build_parser().parse_args([]).compiled_model is True
+    assert build_parser().parse_args(["--compiled_model", "false"]).compiled_model is False
+    kw = dict(max_seq_len=64, max_gpu_num_blocks=32, dtype="float32", page_size=page, max_batch_size=2)
+    assert GenerateText(folder, **kw).engine.runner.graphs is not None
+    assert GenerateText(folder, compiled_model=False, **kw).engine.runner.graphs is None
+
+
+def word_tokenizer(folder, vocab_size):
+    """tokenizer.json with one word "w<i>" per token id, built offline."""
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    tok = Tokenizer(models.WordLevel({f"w{i}": i for i in range(vocab_size)}, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+    tok.save(os.path.join(folder, "tokenizer.json"))
+
+
+@pytest.fixture(scope="module")
+def folder_with_words(tmp_path_factory, gpu_device):
+    """Tiny A with a word-level tokenizer and, as end-of-sequence token, the fourth token that
+    greedy decoding of the test prompt gives: text generation must stop there."""
+    import json
+    folder, page = make_folder(tmp_path_factory, "A", seed=21)
+    cfg, w = plain_llama.read_model_folder(folder)
+    prompt = [7, 1, 30, 200, 11]
+    free = plain_llama.greedy_generate(cfg, w, prompt, 8)
+    stop_at = next(i for i in range(3, 8) if free[i] not in free[:i])
+    cfg["eos_token_id"] = free[stop_at]
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    word_tokenizer(folder, cfg["vocab_size"])
+    return folder, page, prompt, free, stop_at
+
+
+def test_text_completion_matches_the_token_path(folder_with_words):
+    """lite_llama/generate.py:156-177: prompts are encoded, generated from, and decoded without
+    the end-of-sequence token."""
+    from pytriton_llama_amd.generate import GenerateText
+    folder, page, prompt, free, stop_at = folder_with_words
+    gen = GenerateText(folder, max_seq_len=64, max_gpu_num_blocks=64, dtype="float32", page_size=page,
+                       max_batch_size=4)
+    assert gen.tokenizer is not None
+    text = " ".join(f"w{t}" for t in prompt)
+    other = [3, 9, 250]
+    ids, _ = gen.generate([prompt, other], max_gen_len=8, temperature=0.0)
+    assert ids[0] == free[:stop_at + 1]                       # stops with the end-of-sequence token
+    outs = gen.text_completion([text, "w3 w9 w250"], temperature=0.0, max_gen_len=8)
+    words = lambda ts: " ".join(f"w{t}" for t in ts if t != free[stop_at])
+    assert [o["generation"] for o in outs] == [words(ids[0]), words(ids[1])]
+    echoed = gen.text_completion([text], temperature=0.0, max_gen_len=8, echo=True)
+    assert echoed[0]["generation"] == text + " " + words(ids[0])
+    # a limit on new tokens ends the text earlier
+    short = gen.text_completion([text], temperature=0.0, max_gen_len=2)
+    assert short[0]["generation"] == words(free[:2])
+
+
+def test_text_completion_stream_grows_to_the_same_text(folder_with_words):
+    """lite_llama/generate_stream.py:190-216: every yield holds the text so far."""
+    from pytriton_llama_amd.generate import GenerateStreamText
+    folder, page, prompt, free, stop_at = folder_with_words
+    gen = GenerateStreamText(folder, max_seq_len=64, max_gpu_num_blocks=64, dtype="float32",
+                             page_size=page, max_batch_size=4)
+    texts = [" ".join(f"w{t}" for t in prompt), "w3 w9 w250"]
+    whole = gen.text_completion(texts, temperature=0.0, max_gen_len=8)
+    seen = ["", ""]
+    yields = 0
+    for batch in gen.text_completion_stream(texts, temperature=0.0, max_gen_len=8):
+        yields += 1
+        for i, c in enumerate(batch):
+            assert c["generation"].startswith(seen[i])
+            seen[i] = c["generation"]
+    assert yields >= 2 and seen == [w["generation"] for w in whole]
+
+
+@pytest.mark.parametrize("stream", ["true", "false"])
+def test_command_line_with_text_prompts(folder_with_words, stream):
+    """cli.py --prompt (the reference's prompt loop, cli.py:40-66, fed from the command line)."""
+    folder, page, prompt, free, stop_at = folder_with_words
+    text = " ".join(f"w{t}" for t in prompt)
+    out = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "cli.py"), "--checkpoints_dir", folder, "--dtype", "float32",
+         "--temperature", "0", "--max_gen_len", "8", "--max_seq_len", "64", "--max_gpu_num_blocks", "32",
+         "--page_size", str(page), "--stream", stream, "--prompt", text],
+        capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert out.stdout.split() == [f"w{t}" for t in free[:stop_at]]
+    # the prompt loop on standard input
+    out = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "cli.py"), "--checkpoints_dir", folder, "--dtype", "float32",
+         "--temperature", "0", "--max_gen_len", "8", "--max_seq_len", "64", "--max_gpu_num_blocks", "32",
+         "--page_size", str(page)],
+        input=text + "\nexit\n", capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert " ".join(f"w{t}" for t in free[:stop_at]) in out.stdout
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])

@@ -693,7 +693,9 @@ def test_kernels_refuse_cpu_tensors(ops):
     with pytest.raises(ops.KernelError):
         ops.silu_mul(torch.zeros(2, 4))
     with pytest.raises(ops.KernelError):
-        ops.add_rmsnorm(torch.zeros(2, 20000, device="cuda"), None, torch.ones(20000, device="cuda"), 1e-5)
+        ops.add_rmsnorm(torch.zeros(2, 64), None, torch.ones(64), 1e-5)
+    with pytest.raises(ops.KernelError):        # a weight of the wrong length
+        ops.add_rmsnorm(torch.zeros(2, 64, device="cuda"), None, torch.ones(63, device="cuda"), 1e-5)
 
 
 def test_sample_top_p_large_vocabulary_and_ties(ops):

@@ -318,3 +318,122 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(gpu_device):
             err = (got[rid] - want[rid]).abs().max() / float(want[rid].abs().max())
             assert err < 2e-4, (rid, float(err))
         assert runner.manager.paged[0].pool.num_free == 48
+
+
+STATE_ON_DEVICE = {"architectures": ["ToyStateLM"], "vocab_size": 70, "hidden_size": 48, "inner": 96,
+                   "layers": ["state_on_device", "attention", "state_on_device"], "order": [0, 1, 2],
+                   "toy_norm": False, "toy_ffn": False, "heads": 3, "kv_heads": 1, "head_dim": 16,
+                   "initializer_range": 0.25}
+
+
+def state_on_device_plain(model, ids):
+    """Whole-sequence logits of the model above, formulas spelt out, on the CPU."""
+    h, residual = model.embedding.weight.float().cpu()[torch.as_tensor(ids)], None
+    for call in model.schedule:
+        b = model.blocks[call.block]
+        h, residual = plain_llama.add_rms_norm(h, residual, b.input_norm.weight.cpu(), b.input_norm.eps)
+        m = b.mixer
+        if hasattr(m, "decay"):
+            u = h @ m.w.float().cpu().T + m.bias.cpu()
+            s, ys = torch.zeros(u.shape[1]), []
+            for t in range(u.shape[0]):
+                s = m.decay.cpu() * s + u[t]
+                ys.append(s)
+            h = torch.stack(ys)
+        else:
+            S = h.shape[0]
+            qkv = h @ m.qkv.float().cpu().T
+            q = qkv[:, :m.q_size].view(S, m.num_heads, m.head_dim)
+            k = qkv[:, m.q_size:m.q_size + m.kv_size].view(S, m.num_kv_heads, m.head_dim)
+            v = qkv[:, m.q_size + m.kv_size:].view(S, m.num_kv_heads, m.head_dim)
+            cos, sin = plain_llama.rope_cos_sin(m.position.inv_freq_host, torch.arange(S))
+            o = plain_llama.causal_attention(plain_llama.apply_rope(q, cos, sin),
+                                             plain_llama.apply_rope(k, cos, sin), v, m.scale)
+            h = o.reshape(S, -1) @ m.o.float().cpu().T
+        h, residual = plain_llama.add_rms_norm(h, residual, b.post_norm.weight.cpu(), b.post_norm.eps)
+        ff = b.feed_forward
+        gu = h @ ff.gate_up.float().cpu().T
+        I = ff.intermediate_size
+        h = (plain_llama.silu(gu[:, :I]) * gu[:, I:]) @ ff.down.float().cpu().T
+    h, _ = plain_llama.add_rms_norm(h, residual, model.final_norm.weight.cpu(), model.final_norm.eps)
+    return h @ model.head.weight.float().cpu().T
+
+
+def test_toy_state_mixer_keeps_graphs_and_steps_launched_ahead(gpu_device):
+    """A model with fixed-size state per request is replayed as HIP graphs like any other (the
+    rows that pad a step name the padding slot, and the run that records a graph touches no
+    request's state), and its decode steps are launched ahead of their tokens."""
+    from pytriton_llama_amd.config import EngineConfig, build_model
+    from pytriton_llama_amd.engine import Engine, SamplingParams
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_random_weights
+    model = build_model(copy.deepcopy(STATE_ON_DEVICE))
+    assert model.graph_capturable()
+    load_random_weights(model, 4, torch.float32, gpu_device, norm_std=0.1)
+    decay = model.blocks[0].mixer.decay
+    assert float(decay.min()) >= 0.5 and float(decay.max()) <= 0.9       # the part's own init hint
+    g = torch.Generator().manual_seed(8)
+    seqs = {f"r{i}": torch.randint(0, 70, (n,), generator=g).tolist() for i, n in enumerate([40, 21, 57, 33])}
+    want = {rid: state_on_device_plain(model, t) for rid, t in seqs.items()}
+    for steps in (cuttings.tail_decode(seqs, 12), cuttings.portions(seqs), cuttings.mixed(seqs, seed=4)):
+        for st in steps:                         # one wanted place a portion: such steps are replayed
+            for e in st["entries"]:
+                e["want"] = e["want"][-1:]
+        runner = ModelRunner(model, page_size=8, num_pages=40, max_num_seqs=4, max_model_len=64,
+                             use_graphs=True)
+        assert runner.graphs is not None and len(runner.manager.states) == 1
+        from engine_helpers import replay_wanted
+        got = replay_wanted(runner, steps)
+        places = cuttings.wanted_places(steps)
+        for rid in seqs:
+            ref = want[rid][places[rid]]
+            err = (got[rid] - ref).abs().max() / ref.abs().max()
+            assert err < 2e-4, (rid, float(err))
+        assert runner.graphs.buckets and runner.portion_graphs.buckets, "nothing was replayed"
+    # through the engine: steps launched ahead give the tokens of the engine that waits
+    prompts = [t[:9] for t in seqs.values()]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=10)
+    outs = {}
+    for name, kw in (("eager", dict(use_graphs=False)), ("ahead", dict(use_graphs=True, async_decode=True))):
+        eng = Engine(copy.deepcopy(STATE_ON_DEVICE), EngineConfig(
+            dtype="float32", page_size=8, num_pages=40, max_num_seqs=4, max_model_len=64, **kw),
+            random_seed=4, norm_std=0.1)
+        outs[name] = eng.generate(prompts, sp)
+        assert (eng.runner.graphs is not None) == (name == "ahead")
+    assert outs["eager"] == outs["ahead"]
+    for p, o in zip(prompts, outs["eager"]):
+        ref = state_on_device_plain(model, p + o)
+        assert o == [int(ref[len(p) - 1 + i].argmax()) for i in range(len(o))]
+
+
+def test_parts_that_wait_for_the_device_are_never_recorded(gpu_device):
+    from pytriton_llama_amd.config import build_model
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_random_weights
+    model = build_model(copy.deepcopy(HYBRID))
+    assert not model.graph_capturable()
+    load_random_weights(model, 9, torch.float32, gpu_device)
+    runner = ModelRunner(model, page_size=8, num_pages=8, max_num_seqs=2, max_model_len=32, use_graphs=True)
+    assert runner.graphs is None and runner.portion_graphs is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_rmsnorm_part_takes_any_width(gpu_device, dtype):
+    """Rows wider than the kernel's LDS copy (15,000 elements) go through its two-pass form;
+    a width is never refused after the weights have been loaded."""
+    from pytriton_llama_amd.parts import build_part
+    for H in (16384, 20004, 15001):
+        n = build_part("norm", "rmsnorm", size=H, eps=1e-5)
+        g = torch.Generator().manual_seed(H)
+        w = 1 + 0.1 * torch.randn(H, generator=g)
+        n.load({"weight": w}, dtype, gpu_device)
+        x = torch.randn(3, H, generator=g).to(dtype)
+        r = torch.randn(3, H, generator=g).to(dtype)
+        rc = r.clone().cuda()
+        y, res = n.forward(x.cuda(), rc)
+        wy, wr = plain_llama.add_rms_norm(x.float(), r.float(), w, 1e-5)
+        tol = 1e-5 if dtype == torch.float32 else 1e-2
+        torch.testing.assert_close(y.float().cpu(), wy, atol=tol, rtol=tol)
+        torch.testing.assert_close(res.float().cpu(), wr.to(dtype).float(), atol=0, rtol=0)
+        y0, _ = n.forward(x.cuda(), None)
+        torch.testing.assert_close(y0.float().cpu(), plain_llama.rms_norm(x.float(), w, 1e-5), atol=tol, rtol=tol)

@@ -131,3 +131,55 @@ def test_random_weights_depend_on_seed_and_name_only(tmp_path):
     assert torch.equal(t4["model.layers.1.self_attn.q_proj.weight"],
                        t1["model.layers.1.self_attn.q_proj.weight"])
     assert json.load(open(os.path.join(f1, "config.json")))["hidden_size"] == 64
+
+
+def test_init_hints_of_a_part_go_before_the_rule_of_the_kind():
+    """A part may say how its tensors are drawn in the random-weights mode (biases, decay rates,
+    gates are no norm weights); a hint nobody knows is an error."""
+    from pytriton_llama_amd.weights.random_init import random_tensor
+    d = random_tensor(3, "x.decay", (4000,), "vector", 0.02, 0.1, init=("uniform", 0.5, 0.9))
+    assert d.dtype == torch.float32 and 0.5 <= float(d.min()) and float(d.max()) <= 0.9
+    assert abs(float(d.mean()) - 0.7) < 0.01
+    b = random_tensor(3, "x.bias", (4000,), "vector", 0.02, 0.1, init=("normal", 0.0, 0.3))
+    assert abs(float(b.mean())) < 0.03 and abs(float(b.std()) - 0.3) < 0.02
+    c = random_tensor(3, "x.gate", (5, 7), "matrix", 0.02, 0.1, init=("constant", -2.5))
+    assert c.shape == (5, 7) and bool((c == -2.5).all())
+    assert torch.equal(d, random_tensor(3, "x.decay", (4000,), "vector", 0.5, 0.0, init=("uniform", 0.5, 0.9)))
+    n = random_tensor(3, "x.norm", (4000,), "vector", 0.02, 0.1)            # no hint: a norm weight
+    assert abs(float(n.mean()) - 1.0) < 0.01
+    with pytest.raises(ValueError, match="unknown init hint"):
+        random_tensor(3, "x", (4,), "vector", 0.02, 0.1, init=("xavier",))
+    # through a model: the toy mixer's decay rates and bias in a written folder
+    import toy_parts  # noqa: F401
+    from pytriton_llama_amd.config import build_model
+    from pytriton_llama_amd.weights.random_init import random_tensors
+    model = build_model({"architectures": ["ToyStateLM"], "vocab_size": 30, "hidden_size": 16, "inner": 24,
+                         "layers": ["state_on_device"], "toy_norm": False, "toy_ffn": True})
+    drawn = {name: t for name, _, _, t in random_tensors(model, 1, norm_std=0.1)}
+    assert 0.5 <= float(drawn["l0.mixer.decay"].min()) and float(drawn["l0.mixer.decay"].max()) <= 0.9
+    assert abs(float(drawn["l0.mixer.bias"].mean())) < 0.1
+    assert abs(float(drawn["l0.input_norm.weight"].mean()) - 1.0) < 0.1
+
+
+def test_an_untied_checkpoint_without_the_key_is_refused(tmp_path):
+    """config.json without tie_word_embeddings means tied (the reference's default); a file
+    that then brings lm_head.weight is not run with the embedding table in its place."""
+    import json
+    from tiny_configs import tiny
+    from pytriton_llama_amd.config import build_model, read_config_json
+    from pytriton_llama_amd.weights import WeightError, load_weights, write_random_model
+    cfg = tiny("A")[0]
+    cfg["tie_word_embeddings"] = False
+    write_random_model(cfg, str(tmp_path), seed=1, dtype=torch.float32)
+    del cfg["tie_word_embeddings"]
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(cfg, f)
+    model = build_model(read_config_json(str(tmp_path)))
+    with pytest.raises(WeightError) as e:
+        load_weights(model, str(tmp_path), torch.float32, "cpu")
+    assert e.value.unexpected == ["lm_head.weight"]
+    # said in so many words, a tied checkpoint may carry the copy
+    cfg["tie_word_embeddings"] = True
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(cfg, f)
+    load_weights(build_model(read_config_json(str(tmp_path))), str(tmp_path), torch.float32, "cpu")

@@ -43,6 +43,8 @@ class ToyDecayState(Part):
     vector per request (no keys, no pages). It starts from the request's state
     slot and writes it back, so any cutting of a sequence gives the same y."""
 
+    graph_capturable = False         # forward reads q_start and the slots on the host
+
     def __init__(self, hidden_size, decay):
         self.hidden_size, self.decay = hidden_size, decay
 
@@ -70,6 +72,49 @@ class ToyDecayState(Part):
         return y.to(x.dtype)
 
 
+@register_part("mixer", "toy_decay_state_on_device")
+class ToyDecayStateOnDevice(Part):
+    """The same recurrence with a decay rate per channel (a tensor of the checkpoint, drawn
+    between 0.5 and 0.9 in the random-weights mode: no norm weight) and without a word from the
+    device to the host, so that a step can be recorded as a graph. Where a sequence's rows end is
+    read from ctx.q_start on the device: in a recorded step the host's lengths are the upper
+    bounds of the step's size class, and rows past the end are padding that must not move the
+    state."""
+
+    def __init__(self, hidden_size):
+        self.hidden_size = hidden_size
+
+    def cache_spec(self):
+        return StateSpec((self.hidden_size,), torch.float32)
+
+    def param_sources(self):
+        return [ParamSource("w", (self.hidden_size, self.hidden_size)),
+                ParamSource("decay", (self.hidden_size,), "vector", init=("uniform", 0.5, 0.9)),
+                ParamSource("bias", (self.hidden_size,), "vector", init=("normal", 0.0, 0.1))]
+
+    def load(self, tensors, dtype, device):
+        self.w = place(tensors["w"], "matrix", dtype, device)
+        self.decay = place(tensors["decay"], "vector", dtype, device)
+        self.bias = place(tensors["bias"], "vector", dtype, device)
+
+    def forward(self, x, ctx, cache):
+        u = x.float() @ self.w.float().T + self.bias
+        n = ctx.num_seqs
+        first, end = ctx.q_start[:n].long(), ctx.q_start[1:n + 1].long()
+        slots = ctx.state_slots[:n].long()
+        s = cache.state.index_select(0, slots)
+        y = torch.zeros_like(u)
+        for j in range(ctx.max_q_len):
+            row = first + j
+            live = (row < end)[:, None]
+            row = torch.where(live[:, 0], row, first)          # rows past the end: a row of its own
+            s = torch.where(live, self.decay * s + u.index_select(0, row), s)
+            y.index_copy_(0, row, torch.where(live, s, y.index_select(0, row)))
+        if cache.writable:
+            cache.state.index_copy_(0, slots, s)
+        return y.to(x.dtype)
+
+
 @register_part("feed_forward", "toy_relu")
 class ToyRelu(Part):
     def __init__(self, hidden_size, inner):
@@ -92,6 +137,7 @@ class ToyRouted(Part):
     """A feed-forward with routing: router logits in float32, the two best experts of every
     token, their outputs mixed by the softmax over the two logits. Experts are small ReLU
     networks kept in one stacked tensor."""
+    graph_capturable = False         # the rows of an expert are counted on the host
 
     def __init__(self, hidden_size, inner, experts):
         self.hidden_size, self.inner, self.experts = hidden_size, inner, experts
@@ -179,6 +225,8 @@ def build_toy(cfg: ToyConfig) -> CausalLM:
     for i, kind in enumerate(cfg.layers):
         if kind == "state":
             mixer = build_part("mixer", "toy_decay_state", hidden_size=H, decay=cfg.decay)
+        elif kind == "state_on_device":
+            mixer = build_part("mixer", "toy_decay_state_on_device", hidden_size=H)
         else:
             if getattr(cfg, "toy_position", False):
                 pos = build_part("position", "toy_decay", head_dim=cfg.head_dim, strength=0.02)
