@@ -43,6 +43,9 @@ class EngineConfig:
     seed: int = 0
     use_graphs: bool = True                  # replay decode-only steps, and steps that bring one
                                              # portion of one prompt (up to 2,048 tokens), as HIP graphs
+    decode_weight_copies: bool = True        # keep a second copy of the weights in the layout the
+                                             # decode kernels read fastest (doubles the memory the
+                                             # weights take; False on a small card)
     async_decode: bool = True                # launch a decode step before the tokens of the one
                                              # before it have reached the host
 

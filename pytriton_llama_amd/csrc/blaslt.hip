@@ -18,6 +18,10 @@
 namespace {
 
 constexpr size_t WORKSPACE_BYTES = 64u << 20;
+// Plans kept at most. Steps replayed as graphs meet a few dozen shapes; steps launched kernel by
+// kernel bring a new M with every prompt length, so the table is emptied when it is full (the
+// library is only read at call time: a plan may go once its call has returned).
+constexpr size_t MAX_PLANS = 1024;
 
 struct Plan {
   hipblasLtMatmulDesc_t desc = nullptr;
@@ -41,6 +45,14 @@ State& state() {
 }
 
 bool ok(hipblasStatus_t st) { return st == HIPBLAS_STATUS_SUCCESS; }
+
+void drop_plan(Plan& p) {
+  if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+  if (p.b) hipblasLtMatrixLayoutDestroy(p.b);
+  if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
+  if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+  p = Plan();
+}
 
 int make_plan(State& s, Plan& p, int M, int N, int K, long ldx, long ldy, int out_dtype) {
   // Column-major view: y^T [N, M] = W [N, K] x^T [K, M]. W lies as a K x N column-major
@@ -83,16 +95,33 @@ extern "C" int ptl_blaslt_gemm_bf16(void* y, const void* x, const void* w, int M
   State& s = state();
   std::lock_guard<std::mutex> guard(s.lock);
   if (s.handle == nullptr) {
-    if (!ok(hipblasLtCreate(&s.handle))) return PTL_ERR_LAUNCH;
-    if (hipMalloc(&s.workspace, WORKSPACE_BYTES) != hipSuccess) return PTL_ERR_LAUNCH;
+    // the one allocation of these libraries: the library's workspace, at the first call.
+    // Handle and workspace are kept together or not at all, so a call after a failure tries again
+    hipblasLtHandle_t handle = nullptr;
+    void* workspace = nullptr;
+    if (!ok(hipblasLtCreate(&handle))) return PTL_ERR_LAUNCH;
+    if (hipMalloc(&workspace, WORKSPACE_BYTES) != hipSuccess) {
+      (void)hipGetLastError();
+      hipblasLtDestroy(handle);
+      return PTL_ERR_LAUNCH;
+    }
+    s.handle = handle;
+    s.workspace = workspace;
   }
   const Key key(M, N, K, ldx, ldy, out_dtype);
   auto it = s.plans.find(key);
   if (it == s.plans.end()) {
+    if (s.plans.size() >= MAX_PLANS) {
+      for (auto& kv : s.plans) drop_plan(kv.second);
+      s.plans.clear();
+    }
     Plan p;
     const int rc = make_plan(s, p, M, N, K, ldx, ldy, out_dtype);
-    if (rc != PTL_OK) return rc;
-    it = s.plans.emplace(key, std::move(p)).first;
+    if (rc != PTL_OK) {
+      drop_plan(p);
+      return rc;
+    }
+    it = s.plans.emplace(key, p).first;
   }
   return ok(run(s, it->second, y, x, w, stream)) ? PTL_OK : PTL_ERR_LAUNCH;
 }

@@ -1,7 +1,8 @@
 // Shared helpers of the gfx950 kernels: storage-type conversion, wave-level
 // reductions (64-wide wavefronts) and launch checks. Every exported function
 // is extern "C", takes raw device pointers plus a hipStream_t, launches on that
-// stream and returns 0 or a negative error code; it allocates nothing.
+// stream and returns 0 or a negative error code; it allocates nothing (one exception: the
+// library product of blaslt.hip allocates the library's workspace at its first call).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>

@@ -147,6 +147,19 @@ template <int XR, int U> struct GsPack { static constexpr int P = (16 / XR < U) 
 // (measured: packing finer than four rows a block, for one or two rows, gains nothing more)
 static int gs_rows_of(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
+// Where a lane finds its 8 elements of weight row r from column 8 * lg on. Row-major: the rows of
+// a 16-row tile lie K elements apart, and one load instruction of a wave touches 16 pieces of 64
+// bytes. BLOCKED: a second copy of W (made once, for the decode kernels only) cut into tiles of
+// 16 rows x 32 columns, each tile row-major in 1 KB, the tiles of a row block one after the other
+// along K: a load instruction of a wave reads 1 KB in one piece (512 bytes for an 8-row tile), a
+// wave's batch of eight 8 KB. Going from columns k to k + 32 is 512 elements there (GS_KSTEP).
+template <bool BLOCKED>
+__device__ __forceinline__ const bf16_t* gs_row_ptr(const bf16_t* w, int r, int K, int lg) {
+  if (BLOCKED) return w + ((size_t)(r >> 4) * (K >> 5) * 512 + (r & 15) * 32 + 8 * lg);
+  return w + (size_t)r * K + 8 * lg;
+}
+#define GS_KSTEP(BLOCKED) ((BLOCKED) ? 16 : 1)
+
 // The follow-up of a product whose result is added to the residual stream and normalised
 // (ptl_gemm_skinny_add_norm_bf16). The normalisation needs the whole row, which no workgroup
 // has, so the product's kernel does what it can see: s = round_bf16(x W^T) + residual, the
@@ -164,7 +177,7 @@ struct AddNormArgs {
 // the workgroups when N is so small that 16-row tiles would leave CUs without work.
 // ADD_NORM: the epilogue described at AddNormArgs (MT = 1, bfloat16 output).
 // XR: rows of x a packed load takes per block (see gs_from_lane_up); 16: no packing.
-template <int MT, int U, int ROWS, typename TY, bool ADD_NORM = false, int XR = 16>
+template <int MT, int U, int ROWS, typename TY, bool ADD_NORM = false, int XR = 16, bool BLOCKED = false>
 __global__ void __launch_bounds__(1024)
 gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                    int M, int N, int K, long ldx, long ldy, int k_per_wave, AddNormArgs an) {
@@ -173,7 +186,7 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
   const int nwaves = blockDim.x >> 6;
   const int n0 = blockIdx.x * ROWS;
   const bool wrow = ln < ROWS;
-  const bf16_t* wp = w + (size_t)min(n0 + min(ln, ROWS - 1), N - 1) * K + 8 * lg;
+  const bf16_t* wp = gs_row_ptr<BLOCKED>(w, min(n0 + min(ln, ROWS - 1), N - 1), K, lg);
   static_assert(XR == 16 || MT == 1, "packed loads of x are for one tile of rows");
   constexpr int P = GsPack<XR, U>::P;          // blocks a load instruction of x fetches
   const int xrow = ln % XR, xblock = ln / XR;
@@ -195,7 +208,7 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const bool ok = k + 32 * u + 8 * lg < ke && wrow;
-      wf[u].u = ok ? *reinterpret_cast<const uint4*>(wp + k + 32 * u) : make_uint4(0, 0, 0, 0);
+      wf[u].u = ok ? *reinterpret_cast<const uint4*>(wp + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
     }
   };
   auto multiply = [&](GsFrag (&wf)[U], int k) {
@@ -328,7 +341,8 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
 template <int MT, int U, int ROWS>
 static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
                               long ldy, int out_dtype, hipStream_t stream,
-                              const AddNormArgs* an = nullptr) {
+                              const AddNormArgs* an = nullptr, bool blocked = false) {
+  if (blocked && (MT != 1 || K % 32)) return PTL_ERR_ARG;
   const int blocks = (N + ROWS - 1) / ROWS;
   // enough waves to keep every SIMD of 256 CUs busy a few times over, each with
   // at least 256 elements of K to stream
@@ -340,9 +354,11 @@ static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int 
   int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * MT * 64 * 4 * sizeof(float) : 0;
   const int xr = MT == 1 ? gs_rows_of(M) : 16;
-#define GO(TY, AN, XR, args)                                                                         \
-  gemm_skinny_kernel<(XR == 16 ? MT : 1), U, ROWS, TY, AN, XR><<<blocks, waves * 64, lds, stream>>>(   \
+#define GO1(TY, AN, XR, BL, args)                                                                    \
+  gemm_skinny_kernel<(XR == 16 ? MT : 1), U, ROWS, TY, AN, XR, BL><<<blocks, waves * 64, lds, stream>>>( \
       (TY*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, args)
+#define GO(TY, AN, XR, args)                                                                         \
+  if (MT == 1 && blocked) GO1(TY, AN, XR, (MT == 1), args); else GO1(TY, AN, XR, false, args)
 #define BY_ROWS(TY, AN, args)                                                                        \
   switch (xr) {                                                                                      \
     case 4: GO(TY, AN, 4, args); break;                                                              \
@@ -359,6 +375,7 @@ static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int 
   }
 #undef BY_ROWS
 #undef GO
+#undef GO1
   return ptl_launch_status();
 }
 
@@ -368,21 +385,24 @@ static int skinny_rows(int N) { return (N + 15) / 16 <= 160 ? 8 : 16; }
 template <int MT, int U>
 static int launch_skinny(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
                          long ldy, int out_dtype, hipStream_t stream,
-                         const AddNormArgs* an = nullptr) {
+                         const AddNormArgs* an = nullptr, bool blocked = false) {
   // measured on MI355X at K = 2048 and 8192: N = 2048 (128 tiles of 16 rows) gains 10 to 20 %
   // from 8-row tiles, N = 3072 (192 tiles) loses
   if (skinny_rows(N) == 8)
-    return launch_skinny_rows<MT, U, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, an);
-  return launch_skinny_rows<MT, U, 16>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, an);
+    return launch_skinny_rows<MT, U, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, an, blocked);
+  return launch_skinny_rows<MT, U, 16>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, an, blocked);
 }
 
-extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int M, int N, int K,
-                                    long ldx, long ldy, int out_dtype, hipStream_t stream) {
+// w_blocked != 0: ``w`` is the blocked copy of the matrix (see gs_row_ptr; rows padded to a
+// multiple of 16, K a multiple of 32), which the kernels for at most 16 rows of x take.
+extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int w_blocked, int M, int N,
+                                    int K, long ldx, long ldy, int out_dtype, hipStream_t stream) {
   if (M <= 0 || N <= 0) return PTL_OK;
   if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldx < K || ldy < N ||
-      (out_dtype != PTL_DTYPE_F32 && out_dtype != PTL_DTYPE_BF16))
+      (out_dtype != PTL_DTYPE_F32 && out_dtype != PTL_DTYPE_BF16) || (w_blocked && (M > 16 || K % 32)))
     return PTL_ERR_ARG;
-  if (M <= 16) return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
+  if (M <= 16)
+    return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, nullptr, w_blocked != 0);
   if (M <= 32) return launch_skinny<2, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
   return launch_skinny<4, 2>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
 }
@@ -396,16 +416,16 @@ extern "C" int ptl_gemm_skinny_partials(int N) {
 // y = bf16((x W^T + residual) * norm_w), residual <- x W^T + residual, partials[m][j] = sums of
 // squares of the new residual over column blocks (ptl_gemm_skinny_partials(N) of them a row):
 // see AddNormArgs. M <= 16.
-extern "C" int ptl_gemm_skinny_add_norm_bf16(void* y, const void* x, const void* w, void* residual,
-                                             const float* norm_w, float* partials, int M, int N,
-                                             int K, long ldx, long ldy, long ldr,
+extern "C" int ptl_gemm_skinny_add_norm_bf16(void* y, const void* x, const void* w, int w_blocked,
+                                             void* residual, const float* norm_w, float* partials,
+                                             int M, int N, int K, long ldx, long ldy, long ldr,
                                              hipStream_t stream) {
   if (M <= 0 || N <= 0) return PTL_OK;
   if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldx < K || ldy < N || ldr < N || !residual ||
-      !norm_w || !partials)
+      !norm_w || !partials || (w_blocked && K % 32))
     return PTL_ERR_ARG;
   const AddNormArgs an = {(bf16_t*)residual, norm_w, partials, ldr};
-  return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, PTL_DTYPE_BF16, stream, &an);
+  return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, PTL_DTYPE_BF16, stream, &an, w_blocked != 0);
 }
 
 // ===========================================================================
@@ -445,7 +465,7 @@ struct RowScaleArgs {
   float inv_n, eps;
 };
 
-template <int MODE, int U, int ROWS, int XR>
+template <int MODE, int U, int ROWS, int XR, bool BLOCKED>
 __global__ void __launch_bounds__(1024)
 gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                  int M, int N_out, int K, long ldx, long ldy, int k_per_wave, int pair_offset,
@@ -463,8 +483,8 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   const int r1 = group * group_rows + ROWS * tile;
   const int r2 = r1 + pair_offset;
   const bool wrow = ln < ROWS;
-  const bf16_t* wp1 = w + (size_t)(r1 + min(ln, ROWS - 1)) * K + 8 * lg;
-  const bf16_t* wp2 = w + (size_t)(r2 + min(ln, ROWS - 1)) * K + 8 * lg;
+  const bf16_t* wp1 = gs_row_ptr<BLOCKED>(w, r1 + min(ln, ROWS - 1), K, lg);
+  const bf16_t* wp2 = gs_row_ptr<BLOCKED>(w, r2 + min(ln, ROWS - 1), K, lg);
   constexpr int P = GsPack<XR, U>::P;          // blocks a load instruction of x fetches
   const int xrow = ln % XR, xblock = ln / XR;
   const bf16_t* xp = x + (size_t)min(xrow, M - 1) * ldx + 8 * lg + 32 * (xblock < P ? xblock : 0);
@@ -477,8 +497,8 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const bool ok = k + 32 * u + 8 * lg < ke && wrow;
-      w1[u].u = ok ? *reinterpret_cast<const uint4*>(wp1 + k + 32 * u) : make_uint4(0, 0, 0, 0);
-      w2[u].u = ok ? *reinterpret_cast<const uint4*>(wp2 + k + 32 * u) : make_uint4(0, 0, 0, 0);
+      w1[u].u = ok ? *reinterpret_cast<const uint4*>(wp1 + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
+      w2[u].u = ok ? *reinterpret_cast<const uint4*>(wp2 + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
     }
   };
   auto load_x = [&](int k) {
@@ -619,11 +639,13 @@ static int pair_waves(int blocks, int K) {
 // out [M, I] = silu(x Wg^T) * (x Wu^T) for W = [Wg; Wu] of shape [2I, K]; M <= 16, I % 16 == 0
 // partials / n_partials / eps: the normalisation factor of x's rows that is still to be applied
 // (RowScaleArgs; K is the size of the normalised rows); partials == null: none.
-extern "C" int ptl_gate_up_silu_bf16(void* out, const void* x, const void* w, int M, int I, int K,
-                                     long ldx, const float* partials, int n_partials, float eps,
+// w_blocked: as for ptl_gemm_skinny_bf16
+extern "C" int ptl_gate_up_silu_bf16(void* out, const void* x, const void* w, int w_blocked, int M, int I,
+                                     int K, long ldx, const float* partials, int n_partials, float eps,
                                      hipStream_t stream) {
   if (M <= 0 || I <= 0) return PTL_OK;
-  if (M > 16 || I % 16 || K <= 0 || K % 8 || ldx % 8 || ldx < K || (partials && n_partials <= 0))
+  if (M > 16 || I % 16 || K <= 0 || K % 8 || ldx % 8 || ldx < K || (partials && n_partials <= 0) ||
+      (w_blocked && K % 32))
     return PTL_ERR_ARG;
   const RowScaleArgs sc = {partials, n_partials, 1.0f / (float)K, eps};
   const int blocks = I / 16;
@@ -631,21 +653,23 @@ extern "C" int ptl_gate_up_silu_bf16(void* out, const void* x, const void* w, in
   const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
   RopeStoreArgs none = {};
-#define GO(XR)                                                                                        \
-  gemm_pair_kernel<PAIR_SILU, 8, 16, XR><<<blocks, waves * 64, lds, stream>>>(                        \
+#define GO1(XR, BL)                                                                                   \
+  gemm_pair_kernel<PAIR_SILU, 8, 16, XR, BL><<<blocks, waves * 64, lds, stream>>>(                    \
       (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, M, I, K, ldx, I, k_per_wave, I, blocks, 0, none, sc)
+#define GO(XR) if (w_blocked) GO1(XR, true); else GO1(XR, false)
   switch (gs_rows_of(M)) {
     case 4: GO(4); break;
     case 8: GO(8); break;
     default: GO(16); break;
   }
 #undef GO
+#undef GO1
   return ptl_launch_status();
 }
 
 // q_out [M, Hq, D] (row stride ldq); w [(Hq + 2 Hkv) D, K] rows q | k | v; M <= 16, D % 32 == 0
-extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, const void* w, int M,
-                                       int K, long ldx, const int32_t* positions,
+extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, const void* w, int w_blocked,
+                                       int M, int K, long ldx, const int32_t* positions,
                                        const float* inv_freq, const int32_t* slots, void* k_cache,
                                        void* v_cache, int Hq, int Hkv, int D, int page_size,
                                        const float* partials, int n_partials, float eps,
@@ -653,7 +677,7 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
   if (M <= 0) return PTL_OK;
   if (M > 16 || Hq <= 0 || Hkv <= 0 || D <= 0 || D % 32 || K <= 0 || K % 8 || ldx % 8 || ldx < K ||
       ldq < (long)Hq * D || page_size <= 0 || !positions || (slots && (!k_cache || !v_cache)) ||
-      (partials && n_partials <= 0))
+      (partials && n_partials <= 0) || (w_blocked && K % 32))
     return PTL_ERR_ARG;
   const RowScaleArgs sc = {partials, n_partials, 1.0f / (float)K, eps};
   // few heads: 8-column tiles, so that twice as many workgroups share the weight stream
@@ -664,10 +688,11 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
   const int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
   RopeStoreArgs rs = {positions, inv_freq, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, Hq, Hkv, D, page_size};
-#define GO(ROWS, XR)                                                                                  \
-  gemm_pair_kernel<PAIR_ROPE, 8, ROWS, XR><<<blocks, waves * 64, lds, stream>>>(                      \
+#define GO1(ROWS, XR, BL)                                                                             \
+  gemm_pair_kernel<PAIR_ROPE, 8, ROWS, XR, BL><<<blocks, waves * 64, lds, stream>>>(                  \
       (bf16_t*)q_out, (const bf16_t*)x, (const bf16_t*)w, M, Hq * D, K, ldx, ldq, k_per_wave, D / 2,  \
       tiles, D, rs, sc)
+#define GO(ROWS, XR) if (w_blocked) GO1(ROWS, XR, true); else GO1(ROWS, XR, false)
 #define BY_ROWS(ROWS)                                                                                 \
   switch (gs_rows_of(M)) {                                                                            \
     case 4: GO(ROWS, 4); break;                                                                       \
@@ -677,5 +702,6 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
   if (small) { BY_ROWS(8) } else { BY_ROWS(16) }
 #undef BY_ROWS
 #undef GO
+#undef GO1
   return ptl_launch_status();
 }

@@ -84,6 +84,8 @@ class Engine:
         else:
             self.model = build_model(model)
             load_random_weights(self.model, random_seed or 0, ec.dtype, ec.device, norm_std, weight_std)
+        if ec.decode_weight_copies:
+            self.model.make_decode_copies()
         num_pages = ec.num_pages if ec.num_pages is not None else pages_from_memory(self.model, ec)
         self.runner = ModelRunner(self.model, ec.page_size, num_pages, ec.max_num_seqs,
                                   ec.max_model_len, ec.use_graphs)

@@ -68,6 +68,12 @@ class CausalLM:
             libs += tuple(part.kernel_libraries)
         return tuple(dict.fromkeys(libs))
 
+    def make_decode_copies(self) -> int:
+        """Let every part build what it keeps beside its weights for faster decode steps;
+        returns the bytes taken. After the weights are loaded."""
+        return sum(p.make_decode_copies() for p in [self.embedding, *self.blocks, self.final_norm, self.head]
+                   if hasattr(p, "make_decode_copies"))
+
     def graph_capturable(self) -> bool:
         """Whether a step of this model can be recorded as a HIP graph: every part says so."""
         return all(getattr(p, "graph_capturable", True)

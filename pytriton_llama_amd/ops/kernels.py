@@ -209,6 +209,35 @@ def gemm_nt(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
 
 
 SKINNY_MAX_ROWS = 64
+BLOCKED_MAX_ROWS = 16      # rows of x up to which the kernels take the blocked copy of a weight
+
+
+def blocked_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
+    """A second copy of the bfloat16 matrix w [N, K] for the decode kernels: tiles of 16 rows x
+    32 columns, each tile row-major in 1 KB, the tiles of a row block one after the other along
+    K (shape [ceil(N / 16), K / 32, 16, 32]; rows beyond N are zero). A wave's load instruction
+    then reads 1 KB in one piece instead of 16 pieces of 64 bytes that lie a row apart (see
+    gs_row_ptr in csrc/gemm.hip). None when w cannot be cut so (K no multiple of 32)."""
+    if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] % 32 or not w.is_contiguous():
+        return None
+    N, K = w.shape
+    rows = -(-N // 16) * 16
+    if rows != N:
+        w = torch.cat([w, w.new_zeros((rows - N, K))], dim=0)
+    return w.view(rows // 16, 16, K // 32, 32).permute(0, 2, 1, 3).contiguous()
+
+
+def _weight_arg(w: torch.Tensor, blocked: Optional[torch.Tensor], M: int, what: str):
+    """(pointer, flag) of the weight a decode kernel is to read: the blocked copy when one is
+    given and the rows of x are few enough, else w."""
+    if blocked is None or M > BLOCKED_MAX_ROWS:
+        return _ptr(w), 0
+    N, K = w.shape
+    if (blocked.dtype != torch.bfloat16 or not blocked.is_cuda or not blocked.is_contiguous()
+            or tuple(blocked.shape) != (-(-N // 16), K // 32, 16, 32) or K % 32
+            or blocked.data_ptr() % 16):
+        raise KernelError(f"{what}: the blocked copy does not belong to a [{N}, {K}] bfloat16 matrix")
+    return _ptr(blocked), 1
 
 
 def gemm_skinny_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -219,9 +248,11 @@ def gemm_skinny_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
             and w.is_contiguous() and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                blocked: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x @ w.T for at most 64 rows of bfloat16 x, streaming w once
-    (see csrc/gemm.hip). Output bfloat16 or float32."""
+    (see csrc/gemm.hip). Output bfloat16 or float32. ``blocked``: ``blocked_weight(w)``, read
+    instead of w when x has at most 16 rows."""
     _need_gpu(x, w)
     if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
         raise KernelError(f"gemm_skinny: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
@@ -236,7 +267,8 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     ldx = x.stride(0) if M > 1 else max(K, 8)
     lib = library.load("gemm")
-    _check(lib.ptl_gemm_skinny_bf16(_ptr(y), _ptr(x), _ptr(w), M, N, K, ctypes.c_long(ldx),
+    wp, wb = _weight_arg(w, blocked, M, "gemm_skinny")
+    _check(lib.ptl_gemm_skinny_bf16(_ptr(y), _ptr(x), wp, wb, M, N, K, ctypes.c_long(ldx),
                                     ctypes.c_long(N), _F32 if out_dtype == torch.float32 else _BF16,
                                     _stream()), "gemm_skinny")
     return y
@@ -310,7 +342,7 @@ def gemm_skinny_add_norm_fits(x: torch.Tensor, w: torch.Tensor, residual: torch.
 
 
 def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
-                         norm_weight: torch.Tensor, eps: float):
+                         norm_weight: torch.Tensor, eps: float, blocked: Optional[torch.Tensor] = None):
     """The product x @ w.T, the residual sum and the part of an RMSNorm that does not need the
     whole row, in one kernel for at most 16 rows of bfloat16 x (see AddNormArgs in
     csrc/gemm.hip): ``residual`` becomes x @ w.T + residual in place; returned are
@@ -324,8 +356,9 @@ def gemm_skinny_add_norm(x: torch.Tensor, w: torch.Tensor, residual: torch.Tenso
     count = int(lib.ptl_gemm_skinny_partials(N))
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     partials = torch.empty((M, count), dtype=torch.float32, device=x.device)
+    wp, wb = _weight_arg(w, blocked, M, "gemm_skinny_add_norm")
     _check(lib.ptl_gemm_skinny_add_norm_bf16(
-        _ptr(y), _ptr(x), _ptr(w), _ptr(residual), _ptr(norm_weight), _ptr(partials), M, N, K,
+        _ptr(y), _ptr(x), wp, wb, _ptr(residual), _ptr(norm_weight), _ptr(partials), M, N, K,
         ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)), ctypes.c_long(N),
         ctypes.c_long(residual.stride(0) if M > 1 else N), _stream()), "gemm_skinny_add_norm")
     return y, RowScale(partials, N, eps)
@@ -355,7 +388,8 @@ def gate_up_silu_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
     return _fused_x_ok(x, w) and w.shape[0] % 32 == 0
 
 
-def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = None) -> torch.Tensor:
+def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = None,
+                 blocked: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) for w = [Wg; Wu] ([2I, K]) and at most 16 rows of
     bfloat16 x, in one kernel (see csrc/gemm.hip). ``scale``: the factor that the rows
     of x still lack; it is applied to both products."""
@@ -367,7 +401,8 @@ def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = N
     out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
     lib = library.load("gemm")
     pp, count, eps = scale.args(M, K, "gate_up_silu") if scale is not None else _NO_SCALE
-    _check(lib.ptl_gate_up_silu_bf16(_ptr(out), _ptr(x), _ptr(w), M, I, K,
+    wp, wb = _weight_arg(w, blocked, M, "gate_up_silu")
+    _check(lib.ptl_gate_up_silu_bf16(_ptr(out), _ptr(x), wp, wb, M, I, K,
                                      ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)),
                                      pp, count, eps, _stream()),
            "gate_up_silu")
@@ -382,7 +417,7 @@ def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
                    inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                    num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
-                   scale: Optional[RowScale] = None) -> torch.Tensor:
+                   scale: Optional[RowScale] = None, blocked: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q, k, v = x @ w.T (rows of w: q | k | v), q and k rotated, k and v written
     into the cache pages at ``slots``; returns the rotated q [M, Hq, D]. At most 16
     rows of bfloat16 x, head sizes in steps of 32 (see csrc/gemm.hip). ``scale``: the
@@ -413,8 +448,9 @@ def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
     q = torch.empty((M, Hq, D), dtype=torch.bfloat16, device=x.device)
     lib = library.load("gemm")
     pp, count, eps = scale.args(M, K, "qkv_rope_store") if scale is not None else _NO_SCALE
+    wp, wb = _weight_arg(w, blocked, M, "qkv_rope_store")
     _check(lib.ptl_qkv_rope_store_bf16(
-        _ptr(q), ctypes.c_long(Hq * D), _ptr(x), _ptr(w), M, K,
+        _ptr(q), ctypes.c_long(Hq * D), _ptr(x), wp, wb, M, K,
         ctypes.c_long(x.stride(0) if M > 1 else max(K, 8)), _ptr(positions), _ptr(inv_freq),
         _ptr(slots), _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D, int(page_size), pp, count, eps,
         _stream()),

@@ -9,7 +9,7 @@ import torch
 from .. import ops
 from .base import (PagedKVSpec, ParamSource, Part, PendingProduct, PendingScale, as_tensor, place,
                    register_part)
-from .linear import LINEAR_LIBRARIES, linear
+from .linear import LINEAR_LIBRARIES, decode_copy, linear
 
 
 @register_part("mixer", "paged_attention")
@@ -45,6 +45,8 @@ class PagedAttention(Part):
         self.kv_size = self.num_kv_heads * self.head_dim
         self.qkv: Optional[torch.Tensor] = None
         self.o: Optional[torch.Tensor] = None
+        self.qkv_blocked: Optional[torch.Tensor] = None          # decode copies (make_decode_copies)
+        self.o_blocked: Optional[torch.Tensor] = None
         libs = ("attention", "rope") + LINEAR_LIBRARIES
         if self.head_dim % 32 == 0 and self.head_dim <= 128:
             libs += ("attention_prefill",)          # the matrix-core kernel for prompt portions
@@ -74,6 +76,11 @@ class PagedAttention(Part):
         if self.position is not None:
             self.position.load({}, dtype, device)
 
+    def make_decode_copies(self) -> int:
+        self.qkv_blocked, self.o_blocked = decode_copy(self.qkv), decode_copy(self.o)
+        return sum(t.numel() * t.element_size() for t in (self.qkv_blocked, self.o_blocked)
+                   if t is not None)
+
     takes_pending_scale = True
     can_defer_output = True
 
@@ -91,13 +98,13 @@ class PagedAttention(Part):
             # the few rows of a decode step: projection, rotation and cache write in one kernel
             q = ops.qkv_rope_store(x, self.qkv, ctx.positions, rotary,
                                    group.slots if cache.writable else None, cache.k, cache.v,
-                                   Hq, Hkv, D, cache.page_size, scale)
+                                   Hq, Hkv, D, cache.page_size, scale, blocked=self.qkv_blocked)
             out = torch.empty((T, Hq, D), dtype=x.dtype, device=x.device)
             self.attend(out, q, cache, ctx, group)
             if defer_output:
-                return PendingProduct(out.view(T, Hq * D), self.o)
-            return linear(out.view(T, Hq * D), self.o)
-        qkv = linear(x, self.qkv)
+                return PendingProduct(out.view(T, Hq * D), self.o, self.o_blocked)
+            return linear(out.view(T, Hq * D), self.o, blocked=self.o_blocked)
+        qkv = linear(x, self.qkv, blocked=self.qkv_blocked)
         q = qkv[:, :self.q_size].view(T, Hq, D)
         k = qkv[:, self.q_size:self.q_size + self.kv_size].view(T, Hkv, D)
         v = qkv[:, self.q_size + self.kv_size:].view(T, Hkv, D)
@@ -111,7 +118,7 @@ class PagedAttention(Part):
                        cache.page_size)
         out = torch.empty((T, Hq, D), dtype=x.dtype, device=x.device)
         self.attend(out, q, cache, ctx, group)
-        return linear(out.view(T, Hq * D), self.o)
+        return linear(out.view(T, Hq * D), self.o, blocked=self.o_blocked)
 
     # ---- which kernel takes which sequences --------------------------------------
     def decode_splits(self, ctx, n_dec: int, matrix_cores: bool, device) -> int:

@@ -85,11 +85,12 @@ class StateSpec:
 
 
 class PendingProduct:
-    """x @ w.T that has not been computed (see the module text)."""
-    __slots__ = ("x", "w")
+    """x @ w.T that has not been computed (see the module text). ``blocked``: the decode copy
+    of w (parts/linear.py), if the part keeps one."""
+    __slots__ = ("x", "w", "blocked")
 
-    def __init__(self, x: torch.Tensor, w: torch.Tensor):
-        self.x, self.w = x, w
+    def __init__(self, x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Tensor] = None):
+        self.x, self.w, self.blocked = x, w, blocked
 
     @property
     def shape(self):
@@ -97,7 +98,7 @@ class PendingProduct:
 
     def tensor(self) -> torch.Tensor:
         from .linear import linear
-        return linear(self.x, self.w)
+        return linear(self.x, self.w, blocked=self.blocked)
 
 
 class PendingScale:
@@ -143,6 +144,12 @@ class Part:
 
     def load(self, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device) -> None:
         pass
+
+    def make_decode_copies(self) -> int:
+        """Optional: build what the part keeps beside its weights to run decode steps faster
+        (second copies in another layout, say) and return the bytes it took. Called once after
+        the weights are loaded, when the engine is told to spend memory on speed."""
+        return 0
 
 
 PART_KINDS = ("embedding", "norm", "mixer", "feed_forward", "position", "head", "block")

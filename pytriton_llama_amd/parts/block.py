@@ -35,6 +35,10 @@ class PreNormBlock(Part):
         norm (parts/base.py): what the model asks when it runs two blocks in a row."""
         return bool(getattr(self.input_norm, "takes_pending_product", False))
 
+    def make_decode_copies(self) -> int:
+        return sum(p.make_decode_copies() for p in self.children().values()
+                   if hasattr(p, "make_decode_copies"))
+
     @property
     def graph_capturable(self) -> bool:
         return all(getattr(p, "graph_capturable", True) for p in self.children().values())

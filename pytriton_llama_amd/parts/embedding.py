@@ -7,7 +7,7 @@ import torch
 
 from .. import ops
 from .base import ParamSource, Part, place, register_part
-from .linear import LINEAR_LIBRARIES, linear
+from .linear import LINEAR_LIBRARIES, decode_copy, linear
 
 
 @register_part("embedding", "token_embedding")
@@ -44,6 +44,7 @@ class LinearHead(Part):
         self.tied_to = tied_to
         self.weight_name = weight_name
         self._weight: Optional[torch.Tensor] = None
+        self.blocked: Optional[torch.Tensor] = None              # decode copy (make_decode_copies)
 
     @property
     def weight(self) -> torch.Tensor:
@@ -58,5 +59,9 @@ class LinearHead(Part):
         if self.tied_to is None:
             self._weight = place(tensors[self.weight_name], "matrix", dtype, device)
 
+    def make_decode_copies(self) -> int:
+        self.blocked = decode_copy(self.weight)
+        return 0 if self.blocked is None else self.blocked.numel() * self.blocked.element_size()
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return linear(x, self.weight, out_dtype=torch.float32)
+        return linear(x, self.weight, out_dtype=torch.float32, blocked=self.blocked)

@@ -7,7 +7,7 @@ import torch
 
 from .. import ops
 from .base import ParamSource, Part, PendingProduct, PendingScale, as_tensor, place, register_part
-from .linear import LINEAR_LIBRARIES, linear
+from .linear import LINEAR_LIBRARIES, decode_copy, linear
 
 
 @register_part("feed_forward", "swiglu")
@@ -27,6 +27,8 @@ class SwiGLU(Part):
         self.names = (gate_name, up_name, down_name)
         self.gate_up: Optional[torch.Tensor] = None
         self.down: Optional[torch.Tensor] = None
+        self.gate_up_blocked: Optional[torch.Tensor] = None      # decode copies (make_decode_copies)
+        self.down_blocked: Optional[torch.Tensor] = None
 
     def param_sources(self) -> List[ParamSource]:
         g, u, d = self.names
@@ -39,6 +41,11 @@ class SwiGLU(Part):
         self.gate_up = place(torch.cat([tensors[g], tensors[u]], dim=0), "matrix", dtype, device)
         self.down = place(tensors[d], "matrix", dtype, device)
 
+    def make_decode_copies(self) -> int:
+        self.gate_up_blocked, self.down_blocked = decode_copy(self.gate_up), decode_copy(self.down)
+        return sum(t.numel() * t.element_size() for t in (self.gate_up_blocked, self.down_blocked)
+                   if t is not None)
+
     def forward(self, x, defer_output: bool = False):
         scale = None
         if isinstance(x, PendingScale) and ops.gate_up_silu_fits(x.values, self.gate_up):
@@ -46,8 +53,8 @@ class SwiGLU(Part):
         x = as_tensor(x)
         if ops.gate_up_silu_fits(x, self.gate_up):
             # the few rows of a decode step: product and SiLU-multiply in one kernel
-            a = ops.gate_up_silu(x, self.gate_up, scale)
+            a = ops.gate_up_silu(x, self.gate_up, scale, blocked=self.gate_up_blocked)
             if defer_output:
-                return PendingProduct(a, self.down)
-            return linear(a, self.down)
+                return PendingProduct(a, self.down, self.down_blocked)
+            return linear(a, self.down, blocked=self.down_blocked)
         return linear(ops.silu_mul(linear(x, self.gate_up)), self.down)

@@ -21,7 +21,18 @@ SKINNY_ROWS = 8          # rows up to which the skinny kernel takes a bfloat16 p
 SKINNY_ROWS_F32 = 16     # ... when float32 output is wanted (the head)
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def decode_copy(w: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """The second, blocked copy of a weight matrix that the kernels for the few rows of a decode
+    step read faster (ops.blocked_weight); None where there is none to be had (float32, a K that
+    does not divide)."""
+    if w is None or not w.is_cuda or w.dtype != torch.bfloat16:
+        return None
+    return ops.blocked_weight(w)
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           blocked: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``blocked``: decode_copy(w), for the kernels that take it."""
     if not x.is_cuda:
         raise ops.KernelError("linear: tensors must be on the GPU (there is no CPU path)")
     out_dtype = out_dtype or x.dtype
@@ -32,7 +43,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     # measured on MI355X at the 1B shapes: the weight-streaming kernel is level with the
     # library up to 8 rows (and ahead for the vocabulary-sized head); beyond that the library
     if (M <= SKINNY_ROWS or (to_f32 and M <= SKINNY_ROWS_F32)) and ops.gemm_skinny_fits(x, w):
-        return ops.gemm_skinny(x, w, out_dtype)
+        return ops.gemm_skinny(x, w, out_dtype, blocked=blocked)
     if ops.gemm_library_fits(x, w):
         return ops.gemm_library(x, w, out_dtype, checked=True)
     if to_f32:

@@ -36,7 +36,8 @@ class RMSNorm(Part):
             # kernel; the rsqrt factor is left to the part that takes the result
             if (scale_ok and residual is not None
                     and ops.gemm_skinny_add_norm_fits(x.x, x.w, residual, self.weight)):
-                y, scale = ops.gemm_skinny_add_norm(x.x, x.w, residual, self.weight, self.eps)
+                y, scale = ops.gemm_skinny_add_norm(x.x, x.w, residual, self.weight, self.eps,
+                                                    blocked=x.blocked)
                 return PendingScale(y, scale), residual
         x = as_tensor(x)
         y = ops.add_rmsnorm(x, residual, self.weight, self.eps)

@@ -38,6 +38,7 @@ def load_runner(folder, dtype, page_size, num_pages, device="cuda:0", max_num_se
     from pytriton_llama_amd.weights import load_weights
     model = build_model(read_config_json(folder))
     load_weights(model, folder, dtype, device)
+    model.make_decode_copies()                 # as the engine does by default
     return ModelRunner(model, page_size, num_pages, max_num_seqs)
 
 
@@ -89,6 +90,7 @@ def load_graph_runner(folder, dtype, page_size, num_pages, max_model_len, max_nu
     from pytriton_llama_amd.weights import load_weights
     model = build_model(read_config_json(folder))
     load_weights(model, folder, dtype, device)
+    model.make_decode_copies()
     return ModelRunner(model, page_size, num_pages, max_num_seqs, max_model_len=max_model_len,
                        use_graphs=True)
 

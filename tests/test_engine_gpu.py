@@ -69,6 +69,29 @@ def test_mixed_with_page_reuse(cases, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_cuttings_replayed_as_graphs(cases, name, dtype):
+    """The same cuttings with decode steps and single portions replayed as HIP graphs (their
+    padded layouts of a step against the plain model, not against the eager layout): the last
+    tokens one by one, portions of changing size, and the mixed trace. A replayed portion has
+    one wanted place, so only the last row of every entry is asked for."""
+    from engine_helpers import first_wrong_row, load_graph_runner, plain_rows, replay_wanted
+    folder, page, seqs, _ = cases[name]
+    for steps in (cuttings.tail_decode(seqs, 32), cuttings.portions(seqs), cuttings.mixed(seqs, seed=3)):
+        for st in steps:
+            for e in st["entries"]:
+                e["want"] = e["want"][-1:]
+        places = cuttings.wanted_places(steps)
+        want = plain_rows(folder, seqs, places, dtype)
+        runner = load_graph_runner(folder, dtype, page, -(-cuttings.max_live_tokens(steps) // page),
+                                   max_model_len=160, max_num_seqs=4)
+        got = replay_wanted(runner, steps)
+        bad = first_wrong_row(got, want, places, TOL[dtype])
+        assert bad is None, f"config {name} {dtype}: first wrong place (request, position, error) = {bad}"
+        assert runner.graphs.buckets and runner.portion_graphs.buckets
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_first_tokens_of_a_sequence(cases, dtype):
     """Positions 0, 1, 2: one token whole, then one by one from an empty cache."""
     folder, page, seqs, want = cases["B"]

@@ -280,6 +280,59 @@ def test_fused_products_apply_a_row_scale(ops):
     assert (q_plain.float() - q.float()).abs().max() > 0.1
 
 
+@pytest.mark.parametrize("dims", [(8, 2048, 2048, 8192, 32, 8, 64, 16), (1, 2048, 2048, 8192, 32, 8, 64, 16),
+                                  (16, 160, 224, 224, 3, 1, 32, 8), (5, 3072, 3072, 1024, 24, 8, 128, 16),
+                                  (3, 64, 64, 160, 8, 2, 32, 4), (13, 4128, 96, 64, 2, 2, 96, 16),
+                                  (7, 1000, 96, 48, 5, 5, 32, 2)])
+def test_decode_kernels_read_the_blocked_copy_of_a_weight(ops, dims):
+    """The decode kernels with the second, blocked copy of their weights (tiles of 16 rows x 32
+    columns, each in one piece) give bit for bit what they give with the row-major matrix: the
+    same sums in the same order, only fetched from other addresses. Widths that are no multiple
+    of 16 rows (padding), 8- and 16-row tiles, one to sixteen rows of x."""
+    M, H, Kin, I, Hq, Hkv, D, P = dims
+    g = torch.Generator().manual_seed(M * 7 + H)
+    rnd = lambda *s: torch.randn(*s, generator=g)
+    dev = "cuda"
+    x = rnd(M, Kin).to(torch.bfloat16).to(dev)
+    wo = (rnd(H, Kin) / math.sqrt(Kin)).to(torch.bfloat16).to(dev)
+    wgu = (rnd(2 * I, H) / math.sqrt(H)).to(torch.bfloat16).to(dev)
+    wq = (rnd((Hq + 2 * Hkv) * D, H) / math.sqrt(H)).to(torch.bfloat16).to(dev)
+    nw = (1 + 0.1 * rnd(H)).to(dev)
+    res = rnd(M, H).to(torch.bfloat16).to(dev)
+    bo, bgu, bq = ops.blocked_weight(wo), ops.blocked_weight(wgu), ops.blocked_weight(wq)
+    assert bo.shape == (-(-H // 16), Kin // 32, 16, 32)
+    # the layout itself: tile t, column block b holds rows 16 t .. 16 t + 15, columns 32 b .. 32 b + 31
+    t, b = bo.shape[0] - 1, bo.shape[1] - 1
+    rows = wo[16 * t:16 * t + 16, 32 * b:32 * b + 32]
+    assert torch.equal(bo[t, b, :rows.shape[0]], rows) and bool((bo[t, b, rows.shape[0]:] == 0).all())
+    for out_dtype in (torch.bfloat16, torch.float32):
+        assert torch.equal(ops.gemm_skinny(x, wo, out_dtype), ops.gemm_skinny(x, wo, out_dtype, blocked=bo))
+    r1, r2 = res.clone(), res.clone()
+    y1, s1 = ops.gemm_skinny_add_norm(x, wo, r1, nw, 1e-5)
+    y2, s2 = ops.gemm_skinny_add_norm(x, wo, r2, nw, 1e-5, blocked=bo)
+    assert torch.equal(y1, y2) and torch.equal(r1, r2) and torch.equal(s1.partials, s2.partials)
+    assert torch.equal(ops.gate_up_silu(y1, wgu, s1), ops.gate_up_silu(y1, wgu, s1, blocked=bgu))
+    assert torch.equal(ops.gate_up_silu(y1, wgu), ops.gate_up_silu(y1, wgu, blocked=bgu))
+    positions = torch.randint(0, 3000, (M,), generator=g).to(torch.int32).to(dev)
+    inv_freq = plain_llama.rope_inv_freq_default(10000.0, D).to(dev)
+    slots = (torch.randperm(2 * P, generator=g)[:M]).to(torch.int32).to(dev) if M <= 2 * P else None
+    outs = []
+    for blocked in (None, bq):
+        kc = torch.zeros(2, Hkv, P, D, device=dev, dtype=torch.bfloat16)
+        vc = torch.zeros_like(kc)
+        q = ops.qkv_rope_store(y1, wq, positions, inv_freq, slots, kc if slots is not None else None,
+                               vc if slots is not None else None, Hq, Hkv, D, P, s1, blocked=blocked)
+        outs.append((q, kc, vc))
+    for a, b2 in zip(*outs):
+        assert torch.equal(a, b2)
+    # a copy that belongs to another matrix is refused, more rows than the kernels take fall back
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(x, wo, blocked=torch.zeros((bo.shape[0] + 1, *bo.shape[1:]), dtype=torch.bfloat16, device=dev))
+    x20 = rnd(20, Kin).to(torch.bfloat16).to(dev)
+    assert torch.equal(ops.gemm_skinny(x20, wo), ops.gemm_skinny(x20, wo, blocked=bo))
+    assert ops.blocked_weight(rnd(8, 40).to(torch.bfloat16).to(dev)) is None       # K no multiple of 32
+
+
 def _rope_reference(x, positions, inv_freq):
     cos, sin = plain_llama.rope_cos_sin(inv_freq, positions)
     return plain_llama.apply_rope(x, cos, sin)
