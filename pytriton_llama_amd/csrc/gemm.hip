@@ -342,7 +342,7 @@ template <int MT, int U, int ROWS>
 static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
                               long ldy, int out_dtype, hipStream_t stream,
                               const AddNormArgs* an = nullptr, bool blocked = false) {
-  if (blocked && (MT != 1 || K % 32)) return PTL_ERR_ARG;
+  if (blocked && K % 32) return PTL_ERR_ARG;
   const int blocks = (N + ROWS - 1) / ROWS;
   // enough waves to keep every SIMD of 256 CUs busy a few times over, each with
   // at least 256 elements of K to stream
@@ -358,7 +358,7 @@ static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int 
   gemm_skinny_kernel<(XR == 16 ? MT : 1), U, ROWS, TY, AN, XR, BL><<<blocks, waves * 64, lds, stream>>>( \
       (TY*)y, (const bf16_t*)x, (const bf16_t*)w, M, N, K, ldx, ldy, k_per_wave, args)
 #define GO(TY, AN, XR, args)                                                                         \
-  if (MT == 1 && blocked) GO1(TY, AN, XR, (MT == 1), args); else GO1(TY, AN, XR, false, args)
+  if (blocked) GO1(TY, AN, XR, true, args); else GO1(TY, AN, XR, false, args)
 #define BY_ROWS(TY, AN, args)                                                                        \
   switch (xr) {                                                                                      \
     case 4: GO(TY, AN, 4, args); break;                                                              \
@@ -394,17 +394,17 @@ static int launch_skinny(void* y, const void* x, const void* w, int M, int N, in
 }
 
 // w_blocked != 0: ``w`` is the blocked copy of the matrix (see gs_row_ptr; rows padded to a
-// multiple of 16, K a multiple of 32), which the kernels for at most 16 rows of x take.
+// multiple of 16, K a multiple of 32).
 extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int w_blocked, int M, int N,
                                     int K, long ldx, long ldy, int out_dtype, hipStream_t stream) {
   if (M <= 0 || N <= 0) return PTL_OK;
   if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldx < K || ldy < N ||
-      (out_dtype != PTL_DTYPE_F32 && out_dtype != PTL_DTYPE_BF16) || (w_blocked && (M > 16 || K % 32)))
+      (out_dtype != PTL_DTYPE_F32 && out_dtype != PTL_DTYPE_BF16) || (w_blocked && K % 32))
     return PTL_ERR_ARG;
-  if (M <= 16)
-    return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, nullptr, w_blocked != 0);
-  if (M <= 32) return launch_skinny<2, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
-  return launch_skinny<4, 2>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream);
+  const bool bl = w_blocked != 0;
+  if (M <= 16) return launch_skinny<1, 8>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, nullptr, bl);
+  if (M <= 32) return launch_skinny<2, 4>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, nullptr, bl);
+  return launch_skinny<4, 2>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, nullptr, bl);
 }
 
 // How many partial sums a row gets from ptl_gemm_skinny_add_norm_bf16 with N columns.

@@ -209,7 +209,7 @@ def gemm_nt(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
 
 
 SKINNY_MAX_ROWS = 64
-BLOCKED_MAX_ROWS = 16      # rows of x up to which the kernels take the blocked copy of a weight
+BLOCKED_MAX_ROWS = 64      # rows of x up to which the kernels take the blocked copy of a weight
 
 
 def blocked_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
