@@ -7,9 +7,11 @@ A step is one decode step of the whole engine (schedule, model step over the
 paged cache, sampling, bookkeeping) for a batch of requests whose prompts are
 already in the cache. The default run: random weights N(0, 0.02) of the 1B
 shape, batch 8, 2,048-token prompts of seeded uniform-random token ids, greedy
-sampling, EOS ignored. One JSON line is printed: decoded tokens a second at
-batch 8, the prefill of one 2,048-token prompt, the decode step's HBM roofline
-and the decode rates at batch 1 and 64.
+sampling, EOS ignored, 256 timed steps: the contexts grow from 2,048 to 2,304
+tokens while the clock runs (the warm-up steps are taken by a batch of the same
+shape that is thrown away before the timed one goes in). One JSON line is
+printed: decoded tokens a second at batch 8, the prefill of one 2,048-token
+prompt, the decode step's HBM roofline and the decode rates at batch 1 and 64.
 """
 import argparse
 import json
@@ -94,14 +96,33 @@ def mixed_workload(args, cfg, short):
     warm = engine.generate([torch.randint(0, cfg["vocab_size"], (600,), generator=g).tolist()],
                            SamplingParams(temperature=0.0, max_new_tokens=8, ignore_eos=True))
     prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lens]
+    nums = model_numbers(cfg, 2 if short == "bf16" else 4)
     torch.cuda.synchronize()
     t = time.perf_counter()
     steps = 0
-    for p in prompts:
-        engine.add_request(p, sp)
+    ids = [engine.add_request(p, sp) for p in prompts]
+    reqs = [engine.requests[i] for i in ids]
+    # what the steps have to do, counted from what every step computed: the flops of the
+    # products and of the attention, and the bytes a step must read (every weight once, the keys
+    # and values of every sequence it touches once)
+    flops = bytes_read = 0
+    before = [0] * N
+    attn_unit = nums["attn_flops"](1)                      # per (query, key) pair of all layers
     while engine.has_work:
         engine.step()
         steps += 1
+        touched = 0
+        for k, r in enumerate(reqs):
+            now = r.num_computed
+            n = now - before[k]
+            if n > 0:
+                touched += 1
+                flops += nums["linear_flops_per_token"] * n + attn_unit * (n * before[k] + n * (n + 1) // 2)
+                bytes_read += now * nums["kv_bytes_per_token"]
+                before[k] = now
+        if touched:
+            bytes_read += nums["weight_bytes"]
+    flops += nums["head_flops_per_row"] * N * new
     torch.cuda.synchronize()
     dt = time.perf_counter() - t
     out = {"metric": f"mixed continuous batch, {SHAPE_NAMES[args.shape]} shape: {N} requests, prompts 128..4096, "
@@ -109,6 +130,14 @@ def mixed_workload(args, cfg, short):
            "value": round(N * new / dt, 1), "unit": "generated tokens/s", "seconds": round(dt, 3),
            "engine_steps": steps, "prompt_tokens": sum(lens),
            "prompt_tokens_per_s": round(sum(lens) / dt, 1), "preemptions": engine.scheduler.num_preemptions,
+           "tflops": round(flops / dt / 1e12, 1), "flops_frac": round(flops / dt / PEAK_FLOPS[short], 4),
+           "roofline": {"bound": "hbm", "achieved": round(bytes_read / dt / 1e9, 1), "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": round(bytes_read / dt / 1e9 / PEAK_HBM_GBS, 4)},
+           "config": {"model": f"{SHAPE_NAMES[args.shape]} shape, random weights N(0,0.02)",
+                      "layers": cfg["num_hidden_layers"], "hidden_size": cfg["hidden_size"],
+                      "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+                      "head_dim": cfg["head_dim"], "intermediate_size": cfg["intermediate_size"],
+                      "vocab_size": cfg["vocab_size"], "requests": N, "prefill_chunk": 512, "page_size": page},
            "dtype": short, "data": "synthetic", "n_gpus": 1}
     print(json.dumps(out), flush=True)
     return 0
@@ -117,7 +146,7 @@ def mixed_workload(args, cfg, short):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=2048)
@@ -156,12 +185,12 @@ def main():
     page = 16
     # requests whose prompt is in first go on decoding while the others' prompts are computed
     slack = max_batch * -(-S // max(S, 2048)) + 8
-    per_req_pages = -(-(S + W + K + slack) // page)
+    per_req_pages = -(-(S + max(W, K) + slack) // page)
     if args.mixed:
         return mixed_workload(args, cfg, short)
     ec = EngineConfig(dtype=args.dtype, page_size=page, num_pages=per_req_pages * max_batch + 8,
                       max_num_seqs=max_batch, max_num_batched_tokens=max(S, 2048),
-                      max_model_len=S + W + K + slack, seed=0)
+                      max_model_len=S + max(W, K) + slack, seed=0)
     t0 = time.time()
     log(f"building the {cfg['num_hidden_layers']}-layer {args.shape.upper()}-shape model with random weights "
         f"({args.dtype})")
@@ -200,13 +229,27 @@ def main():
         return 0
 
     # ---- decode ---------------------------------------------------------------------
-    def decode_rate(batch, steps, warmup):
-        sp = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + slack - 4, ignore_eos=True)
+    def prefilled(batch, new_tokens):
+        sp = SamplingParams(temperature=0.0, max_new_tokens=new_tokens + slack - 4, ignore_eos=True)
         ids = [engine.add_request(p, sp) for p in prompts(batch)]
         while any(engine.requests[i].num_computed < S for i in ids):
             engine.step()                       # prompts go in, portion by portion
-        for _ in range(warmup):
-            engine.step()
+        return ids
+
+    def drop(ids):
+        for i in ids:
+            engine.abort(i)
+        assert not engine.has_work
+
+    def decode_rate(batch, steps, warmup):
+        """(tokens/s, seconds a step, mean context while timed, GB/s of what a step must read)"""
+        if warmup:
+            ids = prefilled(batch, warmup)      # a batch of the same shape takes the warm-up steps
+            for _ in range(warmup):
+                engine.step()
+            drop(ids)
+        ids = prefilled(batch, steps)
+        first_ctx = [engine.requests[i].num_computed for i in ids]
         sync()
         t = time.perf_counter()
         produced = 0
@@ -216,21 +259,20 @@ def main():
         dt = time.perf_counter() - t
         assert produced == batch * steps, (produced, batch, steps)
         ctx = [engine.requests[i].num_computed for i in ids]
-        for i in ids:
-            engine.abort(i)
-        assert not engine.has_work
-        mean_ctx = sum(ctx) / len(ctx) - steps / 2.0
-        return batch * steps / dt, dt / steps, mean_ctx
+        drop(ids)
+        mean_ctx = (sum(first_ctx) + sum(ctx)) / (2.0 * len(ctx))
+        bytes_step = nums["weight_bytes"] + batch * mean_ctx * nums["kv_bytes_per_token"]
+        return batch * steps / dt, dt / steps, mean_ctx, bytes_step * steps / dt / 1e9
 
-    rate, step_s, mean_ctx = decode_rate(args.batch, K, W)
+    rate, step_s, mean_ctx, achieved = decode_rate(args.batch, K, W)
     log(f"decode batch {args.batch}: {rate:.0f} tok/s, {step_s * 1e3:.3f} ms/step")
-    bytes_step = nums["weight_bytes"] + args.batch * mean_ctx * nums["kv_bytes_per_token"]
-    achieved = bytes_step / step_s / 1e9
     points = {}
     for b in point_batches:
-        r, st, _ = decode_rate(b, max(16, K // 2), max(4, W // 2))
+        r, st, _, gbs = decode_rate(b, max(16, K // 2), max(4, W // 2))
         points[f"decode_b{b}"] = round(r, 1)
-        log(f"decode batch {b}: {r:.0f} tok/s, {st * 1e3:.3f} ms/step")
+        points[f"decode_b{b}_ms_per_step"] = round(st * 1e3, 4)
+        points[f"decode_b{b}_hbm_frac"] = round(gbs / PEAK_HBM_GBS, 4)
+        log(f"decode batch {b}: {r:.0f} tok/s, {st * 1e3:.3f} ms/step, {gbs:.0f} GB/s")
 
     out = {
         "metric": f"decode tokens/s, {SHAPE_NAMES[args.shape]} shape, batch {args.batch}, {S}-token prompts",
@@ -244,7 +286,7 @@ def main():
             "head_dim": cfg["head_dim"], "intermediate_size": cfg["intermediate_size"],
             "vocab_size": cfg["vocab_size"], "tied_embeddings": cfg["tie_word_embeddings"],
             "rope": f"llama3 factor {cfg['rope_scaling']['factor']:g}",
-            "global_batch": args.batch, "seq_len": S, "context_at_timing": round(mean_ctx),
+            "global_batch": args.batch, "seq_len": S, "new_tokens": K, "context_at_timing": round(mean_ctx),
             "page_size": page, "kv_dtype": short, "sampling": "greedy", "parallelism": "single GPU",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
