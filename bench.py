@@ -157,6 +157,9 @@ def main():
     ap.add_argument("--no-probes", action="store_true",
                     help="skip the two probes of the box (streaming read, MFMA loop)")
     ap.add_argument("--prefill-only", action="store_true", help="measure the prefill and stop (for profiles)")
+    ap.add_argument("--prefill-chunk", type=int, default=0, metavar="N",
+                    help="compute a prompt in portions of N tokens, one step each (default: the whole prompt "
+                         "in one step, as the 2,048-token measurement does)")
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES),
                     help="layer sizes: the default 1b is the benchmark; 3b and 8b are the secondary shapes")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
@@ -184,12 +187,14 @@ def main():
     K, W, S = args.steps, args.warmup, args.prompt_len
     page = 16
     # requests whose prompt is in first go on decoding while the others' prompts are computed
-    slack = max_batch * -(-S // max(S, 2048)) + 8
+    slack = max_batch * -(-S // (args.prefill_chunk or max(S, 2048))) + 8
     per_req_pages = -(-(S + max(W, K) + slack) // page)
     if args.mixed:
         return mixed_workload(args, cfg, short)
     ec = EngineConfig(dtype=args.dtype, page_size=page, num_pages=per_req_pages * max_batch + 8,
-                      max_num_seqs=max_batch, max_num_batched_tokens=max(S, 2048),
+                      max_num_seqs=max_batch,
+                      max_num_batched_tokens=args.prefill_chunk or max(S, 2048),
+                      prefill_chunk=args.prefill_chunk or None,
                       max_model_len=S + max(W, K) + slack, seed=0)
     t0 = time.time()
     log(f"building the {cfg['num_hidden_layers']}-layer {args.shape.upper()}-shape model with random weights "
@@ -213,7 +218,8 @@ def main():
                                                                     ignore_eos=True))
             sync()
             t = time.perf_counter()
-            engine.step()                       # the whole prompt in one step, first token sampled
+            while engine.has_work:              # the whole prompt in one step (or portion by portion),
+                engine.step()                   # first token sampled
             sync()
             times.append(time.perf_counter() - t)
             engine.requests.pop(rid, None)
@@ -222,6 +228,8 @@ def main():
         flops = nums["linear_flops_per_token"] * S + nums["attn_flops"](S) + nums["head_flops_per_row"]
         prefill = {"value": round(S / best, 1), "tokens": S, "ms": round(best * 1e3, 3),
                    "frac": round(flops / best / PEAK_FLOPS[short], 4)}
+        if args.prefill_chunk:
+            prefill["portions_of"] = args.prefill_chunk
         log(f"prefill {S} tokens: {best * 1e3:.2f} ms ({S / best:.0f} tok/s)")
 
     if args.prefill_only:
