@@ -114,7 +114,7 @@ def capture_forward(model, storage, ctx, device, pool=None):
     at the same time)."""
     side = torch.cuda.Stream(device=device)
     side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
+    with torch.cuda.stream(side), ops.timed_library_products():
         model.forward(ctx, storage)                   # warm-up outside the capture
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()

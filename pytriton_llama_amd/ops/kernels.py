@@ -6,6 +6,7 @@ raises.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import functools
 from typing import Optional
@@ -304,6 +305,19 @@ def gemm_library(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dty
                                     ctypes.c_long(N), _F32 if out_dtype == torch.float32 else _BF16,
                                     _stream()), "gemm_library")
     return y
+
+
+@contextlib.contextmanager
+def timed_library_products():
+    """Inside, the first ``gemm_library`` call of a shape times the library's proposals for it
+    and keeps the fastest (csrc/blaslt.hip); that call waits for the stream. For the warm-up
+    pass of a step that is then recorded as a graph: such shapes come back with every replay."""
+    lib = library.load("blaslt")
+    lib.ptl_blaslt_set_tuning(1)
+    try:
+        yield
+    finally:
+        lib.ptl_blaslt_set_tuning(0)
 
 
 FUSED_MAX_ROWS = 16

@@ -134,15 +134,20 @@ def test_gemm_skinny(ops, out_dtype, mnk):
                                  (512, 2048, 2048), (777, 1000, 328), (2048, 352, 176)])
 def test_gemm_library(ops, out_dtype, mnk):
     """The library product called directly: against a float64 product, also for rows of x that
-    are a slice of a wider buffer, twice (the second call takes the kept plan)."""
+    are a slice of a wider buffer; the second call takes the kept plan, the third times the
+    library's proposals for the shape and the fourth runs the fastest of them."""
     M, N, K = mnk
     torch.manual_seed(9)
     x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
     w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
     want = (x.double() @ w.double().T).float()
     t = dict(atol=1e-4, rtol=1e-4) if out_dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
-    for _ in range(2):
-        y = ops.gemm_library(x, w, out_dtype)
+    for call in range(4):
+        if call == 2:
+            with ops.timed_library_products():
+                y = ops.gemm_library(x, w, out_dtype)
+        else:
+            y = ops.gemm_library(x, w, out_dtype)
         assert y.dtype == out_dtype and y.shape == (M, N)
         torch.testing.assert_close(y.float(), want, **t)
     wide = torch.randn(M, K + 24, device="cuda").to(torch.bfloat16)
@@ -153,6 +158,35 @@ def test_gemm_library(ops, out_dtype, mnk):
     assert not ops.gemm_library_fits(x.float(), w)
     with pytest.raises(ops.KernelError):
         ops.gemm_library(x.float(), w)
+
+
+def test_gemm_library_times_nothing_while_a_graph_is_recorded(ops):
+    """Timing switched on while a HIP graph is recorded: nothing waits for the stream there (the
+    recording would fail), every replay gives the product, and the call after the recording,
+    which does time the proposals, gives it too."""
+    M, N, K = 48, 264, 520
+    torch.manual_seed(10)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    want = (x.double() @ w.double().T).float()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.gemm_library(x, w)                                   # plan, handle and workspace
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), ops.timed_library_products():
+        ys = [ops.gemm_library(x, w) for _ in range(3)]
+    for _ in range(3):
+        for y in ys:
+            y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for y in ys:
+            torch.testing.assert_close(y.float(), want, atol=2e-2, rtol=2e-2)
+    with ops.timed_library_products():
+        torch.testing.assert_close(ops.gemm_library(x, w).float(), want, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(ops.gemm_library(x, w).float(), want, atol=2e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("mik", [(1, 176, 64), (8, 8192, 2048), (16, 320, 136), (5, 48, 2056)])
