@@ -50,7 +50,8 @@ def test_stage_step(ops):
 
 
 @pytest.mark.parametrize("dtype", DT, ids=IDS)
-@pytest.mark.parametrize("shape", [(5, 72), (3, 2048), (2, 5000), (1, 16)])
+@pytest.mark.parametrize("shape", [(5, 72), (3, 2048), (2, 5000), (1, 16),
+                                   (513, 328), (515, 2048), (600, 3072), (517, 4096)])
 def test_add_rmsnorm(ops, dtype, shape):
     torch.manual_seed(0)
     x = torch.randn(shape, device="cuda").to(dtype)
