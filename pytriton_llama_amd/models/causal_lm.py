@@ -39,6 +39,9 @@ class CausalLM:
         self.schedule = list(schedule)
         self.prefixes = list(prefixes)
         self.ignorable = tuple(ignorable)
+        # called by the loader with the names of the checkpoint's tensors before it asks for
+        # expected_tensors(): for what config.json leaves open and the file settles
+        self.before_load = None
         for call in self.schedule:
             if not 0 <= call.block < len(self.blocks):
                 raise ValueError(f"run order names block {call.block}, there are {len(self.blocks)}")

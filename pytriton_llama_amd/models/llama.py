@@ -75,14 +75,20 @@ def build_llama(cfg: LlamaConfig) -> CausalLM:
     prefixes += [("model.norm.", final_norm), ("lm_head.", head)]
     ignorable = ["*.rotary_emb.inv_freq"]
     if cfg.tie_word_embeddings and cfg.tie_word_embeddings_given:
-        # a checkpoint that says it is tied may still carry the copy. Without the key the model
-        # is tied by default, and a head in the file then means the default is wrong for it: it
-        # is reported as unexpected instead of being dropped silently
+        # a checkpoint that says it is tied may still carry the copy
         ignorable.append("lm_head.weight")
     cache_layers = [b.cache_spec() for b in blocks]
     schedule = [LayerCall(i, i) for i in range(len(blocks))]
-    return CausalLM(cfg, embedding, blocks, final_norm, head, cache_layers, schedule, prefixes,
-                    ignorable)
+    model = CausalLM(cfg, embedding, blocks, final_norm, head, cache_layers, schedule, prefixes,
+                     ignorable)
+    if not cfg.tie_word_embeddings_given:
+        # config.json does not say: tied is the reference's default
+        # (lite_llama/models/model_config.py:30), but a file that brings a head of its own is an
+        # untied model, and running it with the embedding table would give wrong logits quietly
+        def the_file_decides(names):
+            head.tied_to = None if "lm_head.weight" in names else embedding
+        model.before_load = the_file_decides
+    return model
 
 
 register_model("LlamaForCausalLM", LlamaConfig, build_llama, model_type="llama")

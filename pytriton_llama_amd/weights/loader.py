@@ -70,6 +70,8 @@ def load_weights(model, folder: str, dtype: torch.dtype, device) -> None:
     from safetensors import safe_open
 
     files = _tensor_files(folder)
+    if getattr(model, "before_load", None) is not None:
+        model.before_load(set(files))
     expected = model.expected_tensors()
     missing = sorted(n for n in expected if n not in files)
     unexpected = sorted(n for n in files if n not in expected and not model.is_ignorable(n))

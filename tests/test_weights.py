@@ -161,9 +161,9 @@ def test_init_hints_of_a_part_go_before_the_rule_of_the_kind():
     assert abs(float(drawn["l0.input_norm.weight"].mean()) - 1.0) < 0.1
 
 
-def test_an_untied_checkpoint_without_the_key_is_refused(tmp_path):
-    """config.json without tie_word_embeddings means tied (the reference's default); a file
-    that then brings lm_head.weight is not run with the embedding table in its place."""
+def test_without_the_key_the_file_decides_whether_the_head_is_tied(tmp_path):
+    """config.json without tie_word_embeddings means tied (the reference's default) unless the
+    file brings lm_head.weight: then that is the head, never the embedding table in its place."""
     import json
     from tiny_configs import tiny
     from pytriton_llama_amd.config import build_model, read_config_json
@@ -174,10 +174,27 @@ def test_an_untied_checkpoint_without_the_key_is_refused(tmp_path):
     del cfg["tie_word_embeddings"]
     with open(tmp_path / "config.json", "w") as f:
         json.dump(cfg, f)
+    from safetensors.torch import load_file, save_file
+    tensors = load_file(str(tmp_path / "model.safetensors"))
     model = build_model(read_config_json(str(tmp_path)))
+    load_weights(model, str(tmp_path), torch.float32, "cpu")
+    assert model.head.tied_to is None and torch.equal(model.head.weight, tensors["lm_head.weight"])
+    assert not torch.equal(model.head.weight, model.embedding.weight)
+    # the same folder without the head: tied
+    head = tensors.pop("lm_head.weight")
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    model = build_model(read_config_json(str(tmp_path)))
+    load_weights(model, str(tmp_path), torch.float32, "cpu")
+    assert model.head.weight is model.embedding.weight
+    # config.json says untied and the head is absent: an error that names it
+    cfg["tie_word_embeddings"] = False
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(cfg, f)
     with pytest.raises(WeightError) as e:
-        load_weights(model, str(tmp_path), torch.float32, "cpu")
-    assert e.value.unexpected == ["lm_head.weight"]
+        load_weights(build_model(read_config_json(str(tmp_path))), str(tmp_path), torch.float32, "cpu")
+    assert e.value.missing == ["lm_head.weight"]
+    tensors["lm_head.weight"] = head
+    save_file(tensors, str(tmp_path / "model.safetensors"))
     # said in so many words, a tied checkpoint may carry the copy
     cfg["tie_word_embeddings"] = True
     with open(tmp_path / "config.json", "w") as f:
