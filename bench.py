@@ -11,7 +11,10 @@ sampling, EOS ignored, 256 timed steps: the contexts grow from 2,048 to 2,304
 tokens while the clock runs (the warm-up steps are taken by a batch of the same
 shape that is thrown away before the timed one goes in). One JSON line is
 printed: decoded tokens a second at batch 8, the prefill of one 2,048-token
-prompt, the decode step's HBM roofline and the decode rates at batch 1 and 64.
+prompt, the decode step's HBM roofline, the decode rates at batch 1 and 64, and
+(points.generate_call_b8) the tokens a second of one whole generate() call for 8
+short prompts with temperature 0.6 and top_p 0.9, which is how the reference's
+own benchmark measures.
 """
 import argparse
 import json
@@ -340,6 +343,25 @@ def main():
         points[f"decode_b{b}_ms_per_step"] = round(st * 1e3, 4)
         points[f"decode_b{b}_hbm_frac"] = round(gbs / PEAK_HBM_GBS, 4)
         log(f"decode batch {b}: {r:.0f} tok/s, {st * 1e3:.3f} ms/step, {gbs:.0f} GB/s")
+
+    # One whole generate() call as the reference's own benchmark times it (examples/benchmark.py:
+    # short prompts, temperature 0.6, top_p 0.9, 256 new tokens, tokens/s over the whole call),
+    # on the engine that is there; --like-reference B is the same through GenerateText.
+    if args.points and args.batch >= 8 and not args.no_prefill:
+        try:
+            lens = torch.randint(10, 61, (8,), generator=g).tolist()
+            short_prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lens]
+            sp = SamplingParams(temperature=0.6, top_p=0.9, max_new_tokens=256)
+            engine.generate(short_prompts, sp)                             # the warm-up call
+            sync()
+            t = time.perf_counter()
+            made = sum(len(o) for o in engine.generate(short_prompts, sp))
+            dt = time.perf_counter() - t
+            points["generate_call_b8"] = round(made / dt, 1)
+            log(f"generate() call, 8 prompts of 10..60 tokens, 256 new tokens, temperature 0.6, top_p 0.9: "
+                f"{made / dt:.0f} tok/s ({dt * 1e3:.0f} ms; the reference publishes 558 to 620 tok/s at batch 8)")
+        except Exception as e:                                              # (never at the cost of the line)
+            log(f"generate() call not measured: {e!r}")
 
     out = {
         "metric": f"decode tokens/s, {SHAPE_NAMES[args.shape]} shape, batch {args.batch}, {S}-token prompts",
