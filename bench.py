@@ -9,7 +9,10 @@ already in the cache. The default run: random weights N(0, 0.02) of the 1B
 shape, batch 8, 2,048-token prompts of seeded uniform-random token ids, greedy
 sampling, EOS ignored, 256 timed steps: the contexts grow from 2,048 to 2,304
 tokens while the clock runs (the warm-up steps are taken by a batch of the same
-shape that is thrown away before the timed one goes in). One JSON line is
+shape that is thrown away before the timed one goes in; the timed requests end
+with the token of the last timed step, so the engine, which otherwise launches
+every decode step ahead of the tokens of the step before, starts no step inside
+the clock whose tokens nobody takes). One JSON line is
 printed: decoded tokens a second at batch 8, the prefill of one 2,048-token
 prompt, the decode step's HBM roofline, the decode rates at batch 1 and 64, and
 (points.generate_call_b8) the tokens a second of one whole generate() call for 8
@@ -299,16 +302,23 @@ def main():
         return 0
 
     # ---- decode ---------------------------------------------------------------------
-    def prefilled(batch, new_tokens):
-        sp = SamplingParams(temperature=0.0, max_new_tokens=new_tokens + slack - 4, ignore_eos=True)
-        ids = [engine.add_request(p, sp) for p in prompts(batch)]
+    def prefilled(batch, new_tokens, ends_there=False):
+        """``batch`` requests with their prompts in the cache and their first tokens sampled.
+        ``ends_there``: every request ends with the token of decode step number ``new_tokens``
+        from here, as the workload says (N new tokens each); the engine then launches no step
+        ahead of the last one, so the timed steps are all that the GPU does inside the clock."""
+        ids = [engine.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=new_tokens + slack - 4,
+                                                    ignore_eos=True)) for p in prompts(batch)]
         while any(engine.requests[i].num_computed < S for i in ids):
             engine.step()                       # prompts go in, portion by portion
+        if ends_there:
+            for i in ids:                       # (those whose prompt went in first have decoded a few tokens)
+                engine.requests[i].params.max_new_tokens = len(engine.requests[i].output) + new_tokens
         return ids
 
     def drop(ids):
         for i in ids:
-            engine.abort(i)
+            engine.abort(i)                     # (nothing left to stop for a request that has ended)
         assert not engine.has_work
 
     def decode_rate(batch, steps, warmup):
@@ -318,8 +328,9 @@ def main():
             for _ in range(warmup):
                 engine.step()
             drop(ids)
-        ids = prefilled(batch, steps)
-        first_ctx = [engine.requests[i].num_computed for i in ids]
+        ids = prefilled(batch, steps, ends_there=True)
+        reqs = [engine.requests[i] for i in ids]
+        first_ctx = [r.num_computed for r in reqs]
         sync()
         t = time.perf_counter()
         produced = 0
@@ -328,7 +339,8 @@ def main():
         sync()
         dt = time.perf_counter() - t
         assert produced == batch * steps, (produced, batch, steps)
-        ctx = [engine.requests[i].num_computed for i in ids]
+        assert all(r.finish_reason == "length" for r in reqs) and not engine.has_work
+        ctx = [r.num_computed for r in reqs]
         drop(ids)
         mean_ctx = (sum(first_ctx) + sum(ctx)) / (2.0 * len(ctx))
         bytes_step = nums["weight_bytes"] + batch * mean_ctx * nums["kv_bytes_per_token"]
