@@ -278,7 +278,7 @@ def main():
     prefill = None
     if not args.no_prefill:
         times = []
-        for i in range(4):
+        for i in range(8):
             rid = engine.add_request(prompts(1)[0], SamplingParams(temperature=0.0, max_new_tokens=1,
                                                                     ignore_eos=True))
             sync()
