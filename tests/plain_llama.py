@@ -124,21 +124,26 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
 # --------------------------------------------------------------------------
 # attention
 # --------------------------------------------------------------------------
-def causal_attention(q, k, v, scale: float, window: Optional[int] = None):
+def causal_attention(q, k, v, scale: float, window: Optional[int] = None, query_positions=None):
     """q: [S, Hq, D]; k, v: [S, Hkv, D]. Query head a reads key/value head
     a // (Hq//Hkv) (lite_llama/kernels/flashattentionv2.py:108); scores are
     q.k*scale with scale = 1/sqrt(D) (lite_llama/models/llama.py:173), keys
     after the query are masked out (flashattentionv2.py:24,37-38), softmax over
     the keys, then the weighted sum of the values (:40-61,160). ``window`` is
     not in the reference (Llama has none); it is here for the engine's general
-    attention part: a query at p then sees keys p-window+1 .. p."""
-    S, Hq, D = q.shape
+    attention part: a query at p then sees keys p-window+1 .. p.
+    ``query_positions``: q holds only the queries at these positions of the
+    sequence ([R, Hq, D]; the result has the same rows), so that a few rows of
+    a long sequence cost R x S scores instead of S x S."""
+    S = k.shape[0]
+    Hq = q.shape[1]
     Hkv = k.shape[1]
     G = Hq // Hkv
     kk = k.repeat_interleave(G, dim=1)
     vv = v.repeat_interleave(G, dim=1)
     scores = torch.einsum("qhd,khd->hqk", q, kk) * scale
-    qi = torch.arange(S)[:, None]
+    qi = (torch.arange(S) if query_positions is None
+          else torch.as_tensor(query_positions, dtype=torch.long))[:, None]
     ki = torch.arange(S)[None, :]
     mask = ki <= qi
     if window is not None:

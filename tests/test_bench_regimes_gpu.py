@@ -155,10 +155,8 @@ def long_cases(shape_folders):
 @pytest.mark.parametrize("name", ["1b", "3b", "8b"])
 def test_long_contexts_at_real_widths(long_cases, name, dtype, graphs):
     """2,304 tokens (2,272 at once, 32 decoded) and 4,640 tokens (nine portions of 512, 32
-    decoded) through two layers of each shape; in bfloat16 also with the portions and the
-    decoded tokens replayed as HIP graphs (planned for the longest request)."""
-    if graphs and dtype == torch.float32:
-        pytest.skip("graph replays are covered in bfloat16 here and in float32 by the tiny models")
+    decoded) through two layers of each shape, launched kernel by kernel and with the portions
+    and the decoded tokens replayed as HIP graphs (planned for the longest request)."""
     folder, seqs, steps, places, want = long_cases(name)
     pages = (2304 + 4640) // 16 + 2
     if graphs:
@@ -172,13 +170,12 @@ def test_long_contexts_at_real_widths(long_cases, name, dtype, graphs):
 
 @pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
-@pytest.mark.parametrize("name", ["1b", "3b"])
+@pytest.mark.parametrize("name", ["1b", "3b", "8b"])
 def test_many_decoding_rows_at_real_widths(shape_folders, name, dtype, graphs):
     """64 requests of 20 to 120 tokens decoding together at the real widths (with eight kv heads
     the decode attention runs without splits from 32 rows on), beside a prompt of 300 tokens in
-    portions of 100; the rows fall to 9 and below as the requests end."""
-    if graphs and dtype == torch.float32:
-        pytest.skip("graph replays are covered in bfloat16 here and in float32 by the tiny models")
+    portions of 100; the rows fall to 9 and below as the requests end. At the 8B widths the
+    fused decode products run over 4,096 and 14,336 columns."""
     folder = shape_folders(name)
     seqs, steps = many_decoders(SHAPES[name]["vocab_size"], 64, seed=7, long_len=300,
                                 want_prompt_rows="last", lengths=(20, 120), portion=100)

@@ -315,6 +315,51 @@ def test_fused_products_apply_a_row_scale(ops):
     assert (q_plain.float() - q.float()).abs().max() > 0.1
 
 
+def test_qkv_rope_store_with_a_large_row_scale(ops):
+    """Rows whose pending factor is large (a residual stream that is nearly zero: one partial
+    sum of 1e-3 .. 30 over 6,184 columns gives factors of 14 to 930) make q and k values of
+    some hundreds. The kernel rounds the scaled projection to bfloat16 before it rotates, as
+    the separate kernels store it between product and rotation, so an element of the result
+    carries the rounding of both elements of its pair: the bound is half a bfloat16 ulp (at most
+    2^-8 of the value) of x1 and of x2 from before the rotation plus half an ulp of the result,
+    not a share of the element itself, which the rotation can make small. Every element must
+    lie within that bound."""
+    torch.manual_seed(249)
+    M, K, D, Hq, Hkv, P = 13, 6184, 128, 7, 1, 5
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn((Hq + 2 * Hkv) * D, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    partials = torch.logspace(-3, math.log10(30.0), M, device="cuda").view(M, 1).contiguous()
+    scale = ops.RowScale(partials, K, 1e-6)
+    f = torch.rsqrt(partials.sum(dim=1).double() / K + 1e-6)
+    assert float(f.max()) > 900 and float(f.min()) < 20
+    positions = torch.tensor([5000, 0, 0, 5000, 77, 77, 0, 77, 5000, 1, 77, 1, 100000],
+                             dtype=torch.int32, device="cuda")
+    inv_freq = plain_llama.rope_inv_freq_default(500000.0, D).cuda()
+    npage = -(-M // P) + 1
+    slots = torch.randperm(npage * P)[:M].to(torch.int32).cuda()
+    kc = torch.zeros(npage, Hkv, P, D, device="cuda", dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    q = ops.qkv_rope_store(x, w, positions, inv_freq, slots, kc, vc, Hq, Hkv, D, P, scale)
+    full = ((x.double() * f[:, None]) @ w.double().T).cpu()
+    cos, sin = plain_llama.rope_cos_sin(inv_freq.cpu(), positions.cpu())
+
+    def check(got, projected, what, rotated=True):
+        want = plain_llama.apply_rope(projected, cos.double(), sin.double()) if rotated else projected
+        a = projected.abs()
+        pair = a + torch.cat((a[..., D // 2:], a[..., :D // 2]), dim=-1) if rotated else a
+        bound = 2.0 ** -8 * (pair + want.abs() if rotated else pair) + 1e-5 * a.amax(dim=(-2, -1), keepdim=True)
+        over = (got.double() - want).abs() - bound
+        assert float(over.max()) <= 0, f"{what}: {float(over.max()):.3g} beyond the rounding bound"
+        assert float(want.abs().max()) > 300          # the case is about large values
+
+    check(q.cpu(), full[:, :Hq * D].view(M, Hq, D), "q")
+    rows = slots.long().cpu()
+    got_k = kc.permute(0, 2, 1, 3).reshape(npage * P, Hkv, D).cpu()[rows]
+    got_v = vc.permute(0, 2, 1, 3).reshape(npage * P, Hkv, D).cpu()[rows]
+    check(got_k, full[:, Hq * D:(Hq + Hkv) * D].view(M, Hkv, D), "k")
+    check(got_v, full[:, (Hq + Hkv) * D:].view(M, Hkv, D), "v", rotated=False)
+
+
 @pytest.mark.parametrize("dims", [(8, 2048, 2048, 8192, 32, 8, 64, 16), (1, 2048, 2048, 8192, 32, 8, 64, 16),
                                   (16, 160, 224, 224, 3, 1, 32, 8), (5, 3072, 3072, 1024, 24, 8, 128, 16),
                                   (3, 64, 64, 160, 8, 2, 32, 4), (13, 4128, 96, 64, 2, 2, 96, 16),
@@ -604,6 +649,98 @@ def test_attention_prefill_mfma_long(ops):
     """Many key tiles, a prefix in the cache, rows that end inside a block."""
     _attention_case(ops, torch.bfloat16, seq_lens=[1100, 700], q_lens=[777, 300], Hq=4, Hkv=1, D=64,
                     P=16, kernel="mfma128")
+
+
+def _hot_keys(dk, kc, bt, P, seq, places, value=2.0):
+    """Key ``places[h]`` of kv head h of sequence ``seq`` becomes ``value`` in every element, in
+    the pages and in the dense copy: a query of the same direction then reads that key alone."""
+    D = kc.shape[-1]
+    for h, pos in enumerate(places):
+        kc[int(bt[seq, pos // P]), h, pos % P] = value
+        dk[seq][pos, h] = torch.full((D,), value)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("keys", [8200, 16400])
+def test_attention_decode_long_contexts(ops, D, keys):
+    """Eight decoded rows over up to 8,200 and 16,400 keys with 32 heads on 8 kv heads, cut into
+    the splits the attention part plans for such a step. In every group of four heads, two
+    queries point at one key each (the first key, the last, both sides of a page's and of a
+    split's edge, ...), so that a tile that is dropped or read twice changes the whole row, and
+    two are random with scores spread over about three, so that the sums over all tiles count."""
+    from types import SimpleNamespace
+
+    from pytriton_llama_amd.parts.attention import PagedAttention
+    Hq, Hkv, P = 32, 8, 16
+    G = Hq // Hkv
+    seq_lens = [keys, keys - 7, keys - 16, keys // 2 + 1, keys - 1, 4100, keys, keys - 33]
+    n = len(seq_lens)
+    part = PagedAttention(hidden_size=Hq * D, num_heads=Hq, num_kv_heads=Hkv, head_dim=D)
+    splits = part.decode_splits(SimpleNamespace(ctx_lens=seq_lens), n, True, torch.device("cuda", 0))
+    assert splits >= 4, "the case is meant to run with several splits"
+    kc, vc, bt, dk, dv = _paged_setup(seq_lens, [1] * n, Hkv, D, P, torch.bfloat16, seed=keys + D)
+    g = torch.Generator().manual_seed(5)
+    q = (3.0 * torch.randn(n, Hq, D, generator=g)).to(torch.bfloat16)
+    per_split = -(-seq_lens[0] // splits)
+    special = [0, 1, P - 1, P, 127, 128, per_split - 1, per_split, 2 * per_split + 1, 4095, 4096]
+    for i, s in enumerate(seq_lens):
+        places = [(special[(i * Hkv + h) % len(special)] if (i + h) % 3 else s - 1 - h) % s
+                  for h in range(Hkv)]
+        _hot_keys(dk, kc, bt, P, i, places)
+        q[i, 0::G] = 2.0
+        q[i, 1::G] = 2.0
+    dev = "cuda"
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    out = torch.zeros(n, Hq, D, dtype=torch.bfloat16, device=dev)
+    scale = 1.0 / math.sqrt(D)
+    ops.attention_decode(out, q.to(dev), kc.to(dev), vc.to(dev), i32(list(range(n + 1))),
+                         i32(seq_lens), bt.to(dev), n, scale, 0, splits, matrix_cores=True)
+    for i, s in enumerate(seq_lens):
+        want = plain_llama.causal_attention(q[i:i + 1].float(), dk[i], dv[i], scale,
+                                            query_positions=[s - 1])[0]
+        got = out[i].float().cpu()
+        # the rows that point at one key return its value
+        assert float(want[0::G].abs().max()) > 0.5
+        err = float((got - want).abs().max()) / float(want.abs().max())
+        assert err < 2e-2, f"sequence {i} ({s} keys, {splits} splits): error {err:.3g} of the largest value"
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("prefix,rows", [(14336, 2048), (8192, 8192)])
+def test_attention_prefill_mfma_long_prefix(ops, D, prefix, rows):
+    """A portion of 2,048 rows behind 14,336 keys in the cache (one workgroup a 64-row block by
+    the plan for 32 heads) and one of 8,192 rows behind 8,192 (128-row blocks, the list shared
+    by fewer workgroups than blocks), with the block size and workgroups that the plan gives
+    and the work list the engine builds. Compared for the first, a middle and the last 128 rows;
+    one query head a group points at one far key, the others are random with wide scores."""
+    from pytriton_llama_amd.engine.batch import work_items
+    Hq, Hkv, P = 32, 8, 16
+    G = Hq // Hkv
+    total = prefix + rows
+    kc, vc, bt, dk, dv = _paged_setup([total], [rows], Hkv, D, P, torch.bfloat16, seed=prefix + D)
+    g = torch.Generator().manual_seed(6)
+    q = (3.0 * torch.randn(rows, Hq, D, generator=g)).to(torch.bfloat16)
+    q[:, 0::G] = 2.0
+    _hot_keys(dk, kc, bt, P, 0, [0, 15, 16, 4095, 8192, prefix - 1, prefix, prefix + 5])
+    n64, n128 = -(-rows // 64), -(-rows // 128)
+    block_rows, groups = ops.attention_prefill_mfma_plan(torch.device("cuda", 0), Hq, D, n64, n128)
+    if rows == 8192:
+        assert block_rows == 128 and groups < n128, "the case is meant to share the list"
+    ws, wo = work_items([rows], [total], 0, block_rows)
+    dev = "cuda"
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    out = torch.zeros(rows, Hq, D, dtype=torch.bfloat16, device=dev)
+    scale = 1.0 / math.sqrt(D)
+    ops.attention_prefill_mfma(out, q.to(dev), kc.to(dev), vc.to(dev), i32([0, rows]), i32([total]),
+                               bt.to(dev), torch.from_numpy(ws).to(dev), torch.from_numpy(wo).to(dev),
+                               scale, 0, block_rows, groups)
+    out = out.float().cpu()
+    for lo in (0, (rows // 2 // 128) * 128 - 64, rows - 128):
+        sel = list(range(lo, lo + 128))
+        want = plain_llama.causal_attention(q[sel].float(), dk[0], dv[0], scale,
+                                            query_positions=[prefix + r for r in sel])
+        err = float((out[sel] - want).abs().max()) / float(want.abs().max())
+        assert err < 2e-2, f"rows {lo}..{lo + 127} behind {prefix} keys: error {err:.3g} of the largest value"
 
 
 @pytest.mark.parametrize("kernel", ["decode", "decode_mfma", "mfma", "mfma128"])

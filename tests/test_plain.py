@@ -228,6 +228,12 @@ def test_attention_invariants():
     # a window of S is no window; a window of 1 returns v
     torch.testing.assert_close(pl.causal_attention(q, k, v, D ** -0.5, window=S), out)
     torch.testing.assert_close(pl.causal_attention(q, k, v, D ** -0.5, window=1), v)
+    # a few query rows alone are the same rows of the whole (with and without a window)
+    rows = [0, 3, 4, 11]
+    for window in (None, 5):
+        whole = pl.causal_attention(q, k, v, D ** -0.5, window=window)
+        some = pl.causal_attention(q[rows], k, v, D ** -0.5, window=window, query_positions=rows)
+        torch.testing.assert_close(some, whole[rows])
 
 
 def test_mha_without_rotation_is_nn_multihead_attention():
