@@ -46,6 +46,12 @@ class EngineConfig:
     decode_weight_copies: bool = True        # keep a second copy of the weights in the layout the
                                              # decode kernels read fastest (doubles the memory the
                                              # weights take; False on a small card)
+    timed_library_products: bool = True      # recorded steps run, for each shape of a library matrix
+                                             # product, the fastest of the library's algorithms by a
+                                             # timing at recording (checked against the first one's
+                                             # result). Which one wins can differ between processes,
+                                             # and with it the last bit of bfloat16 results; False:
+                                             # always the library's first, the same bits every time
     async_decode: bool = True                # launch a decode step before the tokens of the one
                                              # before it have reached the host
 

@@ -108,27 +108,31 @@ class _Bucket:
         return self.np[a:a + k]
 
 
-def capture_forward(model, storage, ctx, device, pool=None):
+def capture_forward(model, storage, ctx, device, pool=None, timed_products: bool = True):
     """(graph, logits) of one forward pass over ``ctx``, whose tensors are static buffers.
     ``pool``: the memory pool the graph's tensors come from (shared by graphs that never run
-    at the same time)."""
+    at the same time). ``timed_products``: the library's matrix products of the step run the
+    proposal that a timing of their shape keeps (timed in the warm-up pass, recorded with the
+    choice); False: the library's first proposal, as in steps launched kernel by kernel."""
     side = torch.cuda.Stream(device=device)
     side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side), ops.timed_library_products():
+    with torch.cuda.stream(side), ops.timed_library_products(timed_products):
         model.forward(ctx, storage)                   # warm-up outside the capture
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, pool=pool):
+    with torch.cuda.graph(graph, pool=pool), ops.timed_library_products(timed_products):
         logits = model.forward(ctx, storage)
     return graph, logits
 
 
 class DecodeGraphs:
-    def __init__(self, model, manager, storage, max_model_len: int, device, pool=None):
+    def __init__(self, model, manager, storage, max_model_len: int, device, pool=None,
+                 timed_products: bool = True):
         self.model, self.manager, self.storage = model, manager, storage
         self.device = device
         self.pool = pool
+        self.timed_products = timed_products
         self.max_model_len = int(max_model_len)
         self.width = -(-self.max_model_len // manager.page_size)
         self.sizes = bucket_sizes(manager.max_num_seqs)
@@ -155,7 +159,8 @@ class DecodeGraphs:
         # the split of the decode attention is fixed at capture: plan it for the longest context
         b.ctx.ctx_lens = [self.max_model_len] * b.size
         b.ctx.max_ctx_len = self.max_model_len
-        b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device, self.pool)
+        b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device, self.pool,
+                                            self.timed_products)
 
     def step(self, entries: Sequence[StepEntry], token_feed=None) -> torch.Tensor:
         """Logits [wanted, vocab] of a step whose entries all bring one token.
@@ -296,10 +301,12 @@ class PortionGraphs:
     """Steps of single-token entries (any number up to the largest decode bucket, also none)
     and exactly one entry of 2 to 2,048 tokens with at most one wanted place."""
 
-    def __init__(self, model, manager, storage, max_model_len: int, device, pool=None):
+    def __init__(self, model, manager, storage, max_model_len: int, device, pool=None,
+                 timed_products: bool = True):
         self.model, self.manager, self.storage = model, manager, storage
         self.device = device
         self.pool = pool
+        self.timed_products = timed_products
         self.max_model_len = int(max_model_len)
         self.width = -(-self.max_model_len // manager.page_size)
         self.sizes = list(PORTION_BUCKETS)
@@ -395,7 +402,7 @@ class PortionGraphs:
             slot_of[:] = m.padding_slot
             b.dev.copy_(b.host, non_blocking=True)
             b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device,
-                                                self.pool)
+                                                self.pool, self.timed_products)
             slot_of[:] = real
             b.copied = torch.cuda.Event()
         b.dev.copy_(b.host, non_blocking=True)

@@ -34,18 +34,65 @@ def pages_that_fit(usable_bytes: int, bytes_per_page: int, state_bytes: int, cap
     return int(n)
 
 
+def graph_pool_bytes(model, engine: EngineConfig) -> int:
+    """Memory the recorded steps' shared pool is allowed for when the cache is sized from free
+    memory: the intermediate results of the largest step that is recorded (a portion of up to
+    2,048 tokens beside max_num_seqs decoding rows) and its float32 logits. Nothing when steps
+    are not recorded."""
+    if not (engine.use_graphs and model.graph_capturable()):
+        return 0
+    from .graphs import PORTION_BUCKETS
+    tokens = min(PORTION_BUCKETS[-1], engine.max_num_batched_tokens) + engine.max_num_seqs
+    return tokens * model.widest_step_row_bytes() + (engine.max_num_seqs + 1) * model.vocab_size * 4
+
+
 def pages_from_memory(model, engine: EngineConfig) -> int:
     """Pages that fit into gpu_memory_fraction of the device after the weights
     are loaded (the reference: (total*0.9 - peak - non_torch) // bytes per block,
-    lite_llama/executor/mem_manager.py:44-60,98-110), less what the state pools take."""
+    lite_llama/executor/mem_manager.py:44-60,98-110), less what the state pools and the
+    recorded steps' memory pool take."""
     probe = CacheManager(model.cache_layers, engine.page_size, 1, engine.max_num_seqs)
     per_page = CacheStorage.bytes_per_page(probe, engine.dtype)
-    fixed = CacheStorage.state_bytes(probe, engine.dtype)
+    fixed = CacheStorage.state_bytes(probe, engine.dtype) + graph_pool_bytes(model, engine)
     free, total = torch.cuda.mem_get_info(torch.device(engine.device))
     usable = int(total * engine.gpu_memory_fraction) - (total - free)
     # no request can use more than max_model_len, and max_num_seqs of them may live
     cap = engine.max_num_seqs * (-(-engine.max_model_len // engine.page_size))
     return pages_that_fit(usable, per_page, fixed, cap)
+
+
+def decode_copies_fit(copies_bytes: int, largest_copy_bytes: int, free_bytes: int,
+                      keep_free_bytes: int) -> bool:
+    """Whether the second copies of the weights for decode steps may be made: they take
+    ``copies_bytes`` for good and, while one is built, its size once more; ``keep_free_bytes``
+    must remain for the cache."""
+    return copies_bytes + largest_copy_bytes + keep_free_bytes <= free_bytes
+
+
+def make_decode_copies_if_room(model, device, keep_free_bytes: int) -> bool:
+    """Build the parts' decode copies unless they would not leave ``keep_free_bytes`` of device
+    memory; says so on stderr when it leaves them out (the model then runs its decode steps
+    from the row-major weights, somewhat slower)."""
+    copies, largest = model.decode_copy_bytes()
+    free, _ = torch.cuda.mem_get_info(torch.device(device))
+    if not decode_copies_fit(copies, largest, free, keep_free_bytes):
+        import sys
+        print(f"[pytriton_llama_amd] no second copies of the weights for decode steps: they need "
+              f"{(copies + largest) >> 20} MiB beside {keep_free_bytes >> 20} MiB for the cache, "
+              f"{free >> 20} MiB are free (decode_weight_copies=False says the same without trying)",
+              file=sys.stderr, flush=True)
+        return False
+    model.make_decode_copies()
+    return True
+
+
+def cache_floor_bytes(model, engine: EngineConfig) -> int:
+    """The least the cache must get: the pages the engine was told to have, or those of one
+    request of max_model_len tokens, plus the state pools and the recorded steps' pool."""
+    probe = CacheManager(model.cache_layers, engine.page_size, 1, engine.max_num_seqs)
+    pages = engine.num_pages if engine.num_pages is not None else -(-engine.max_model_len // engine.page_size)
+    return (pages * CacheStorage.bytes_per_page(probe, engine.dtype)
+            + CacheStorage.state_bytes(probe, engine.dtype) + graph_pool_bytes(model, engine))
 
 
 class _Launched:
@@ -85,10 +132,10 @@ class Engine:
             self.model = build_model(model)
             load_random_weights(self.model, random_seed or 0, ec.dtype, ec.device, norm_std, weight_std)
         if ec.decode_weight_copies:
-            self.model.make_decode_copies()
+            make_decode_copies_if_room(self.model, ec.device, cache_floor_bytes(self.model, ec))
         num_pages = ec.num_pages if ec.num_pages is not None else pages_from_memory(self.model, ec)
         self.runner = ModelRunner(self.model, ec.page_size, num_pages, ec.max_num_seqs,
-                                  ec.max_model_len, ec.use_graphs)
+                                  ec.max_model_len, ec.use_graphs, ec.timed_library_products)
         eos = getattr(self.model.config, "eos_token_ids", ())
         self.scheduler = Scheduler(self.runner.manager, ec.max_num_seqs, ec.max_num_batched_tokens,
                                    ec.prefill_chunk, ec.max_model_len, eos)

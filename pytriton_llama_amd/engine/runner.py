@@ -21,7 +21,8 @@ class ModelRunner:
     around it (lite_llama/executor/model_executor.py:261-320)."""
 
     def __init__(self, model, page_size: int, num_pages, max_num_seqs: int,
-                 max_model_len: Optional[int] = None, use_graphs: bool = False):
+                 max_model_len: Optional[int] = None, use_graphs: bool = False,
+                 timed_library_products: bool = True):
         if model.dtype is None:
             raise RuntimeError("load the model's weights before making a runner")
         self.model = model
@@ -38,9 +39,9 @@ class ModelRunner:
             from .graphs import DecodeGraphs, PortionGraphs
             pool = torch.cuda.graph_pool_handle()
             self.graphs = DecodeGraphs(model, self.manager, self.storage, max_model_len, self.device,
-                                       pool)
+                                       pool, timed_library_products)
             self.portion_graphs = PortionGraphs(model, self.manager, self.storage, max_model_len,
-                                                self.device, pool)
+                                                self.device, pool, timed_library_products)
 
     def admit(self, request: Hashable) -> None:
         slot = self.manager.admit(request)

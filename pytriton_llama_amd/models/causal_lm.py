@@ -11,6 +11,13 @@ import torch
 from ..parts.base import ParamSource, Part, as_tensor, run_norm
 
 
+def _numel(shape) -> int:
+    n = 1
+    for d in shape:
+        n *= int(d)
+    return n
+
+
 @dataclass(frozen=True)
 class LayerCall:
     """One entry of the run order: run ``block`` with cache layer
@@ -76,6 +83,28 @@ class CausalLM:
         returns the bytes taken. After the weights are loaded."""
         return sum(p.make_decode_copies() for p in [self.embedding, *self.blocks, self.final_norm, self.head]
                    if hasattr(p, "make_decode_copies"))
+
+    def decode_copy_bytes(self) -> Tuple[int, int]:
+        """(bytes the decode copies of all parts take at most, bytes of the largest of them):
+        every matrix of the checkpoint once more in the engine dtype; nothing for an engine
+        dtype the decode kernels keep no copies for."""
+        if self.dtype != torch.bfloat16:
+            return 0, 0
+        sizes = [2 * _numel(src.shape) for _, src in self.expected_tensors().values()
+                 if src.kind == "matrix"]
+        return sum(sizes), max(sizes, default=0)
+
+    def widest_step_row_bytes(self) -> int:
+        """Bytes of intermediate results one token of a step leaves in the widest block at most
+        (every matrix product's output row, in the engine dtype, twice over for the
+        element-wise results between them): what a recorded step's memory pool is sized by."""
+        size = 4 if self.dtype == torch.float32 else 2
+        widest = 0
+        for block in self.blocks:
+            parts = block.children().values() if hasattr(block, "children") else [block]
+            rows = sum(src.shape[0] for p in parts for src in p.param_sources() if src.kind == "matrix")
+            widest = max(widest, rows)
+        return 2 * widest * size
 
     def graph_capturable(self) -> bool:
         """Whether a step of this model can be recorded as a HIP graph: every part says so."""

@@ -284,11 +284,15 @@ def gemm_library_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+_timed_products = False        # inside ``timed_library_products``
+
+
 def gemm_library(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                  checked: bool = False) -> torch.Tensor:
     """y = x @ w.T by hipBLASLt, called directly with the descriptors and the algorithm of
     the shape kept from its first call (see csrc/blaslt.hip). Output bfloat16 or float32.
-    ``checked``: the caller has just asked ``gemm_library_fits``."""
+    ``checked``: the caller has just asked ``gemm_library_fits``. The library's first proposal
+    runs, except inside ``timed_library_products``."""
     _need_gpu(x, w)
     if not checked and not gemm_library_fits(x, w):
         raise KernelError("gemm_library: needs bfloat16 x [M, K] and w [N, K] with K a multiple of 8 "
@@ -303,21 +307,34 @@ def gemm_library(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dty
     lib = library.load("blaslt")
     _check(lib.ptl_blaslt_gemm_bf16(_ptr(y), _ptr(x), _ptr(w), M, N, K, ctypes.c_long(ldx),
                                     ctypes.c_long(N), _F32 if out_dtype == torch.float32 else _BF16,
-                                    _stream()), "gemm_library")
+                                    1 if _timed_products else 0, _stream()), "gemm_library")
     return y
 
 
 @contextlib.contextmanager
-def timed_library_products():
-    """Inside, the first ``gemm_library`` call of a shape times the library's proposals for it
-    and keeps the fastest (csrc/blaslt.hip); that call waits for the stream. For the warm-up
-    pass of a step that is then recorded as a graph: such shapes come back with every replay."""
-    lib = library.load("blaslt")
-    lib.ptl_blaslt_set_tuning(1)
+def timed_library_products(on: bool = True):
+    """Inside, ``gemm_library`` runs the proposal of the library that a timing of the shape
+    kept: the first such call of a shape times the library's proposals on its own operands
+    (it waits for the stream; not while the stream is captured) and keeps the fastest whose
+    result agrees with the first proposal's (csrc/blaslt.hip). For the warm-up pass and the
+    recording of a step that is replayed as a graph: such shapes come back with every replay.
+    Outside, every call runs the library's first proposal, whatever was timed. ``on=False``:
+    no effect (for callers that pass a switch on)."""
+    global _timed_products
+    before = _timed_products
+    _timed_products = bool(on) or before
     try:
         yield
     finally:
-        lib.ptl_blaslt_set_tuning(0)
+        _timed_products = before
+
+
+def library_product_choice(M: int, N: int, K: int, ldx: int, out_dtype: torch.dtype = torch.bfloat16) -> int:
+    """The proposal kept for a shape by its timing (0 = the library's first), -1 if the shape
+    has not been timed."""
+    lib = library.load("blaslt")
+    return int(lib.ptl_blaslt_timed_choice(int(M), int(N), int(K), ctypes.c_long(int(ldx)), ctypes.c_long(int(N)),
+                                           _F32 if out_dtype == torch.float32 else _BF16))
 
 
 FUSED_MAX_ROWS = 16

@@ -83,7 +83,7 @@ TOL = {torch.float32: 2e-5, torch.bfloat16: 4e-2}
 
 
 def load_graph_runner(folder, dtype, page_size, num_pages, max_model_len, max_num_seqs=8,
-                      device="cuda:0"):
+                      device="cuda:0", timed_library_products=True):
     """A runner that replays decode steps and single-portion steps as HIP graphs."""
     from pytriton_llama_amd.config import build_model, read_config_json
     from pytriton_llama_amd.engine.runner import ModelRunner
@@ -92,7 +92,7 @@ def load_graph_runner(folder, dtype, page_size, num_pages, max_model_len, max_nu
     load_weights(model, folder, dtype, device)
     model.make_decode_copies()
     return ModelRunner(model, page_size, num_pages, max_num_seqs, max_model_len=max_model_len,
-                       use_graphs=True)
+                       use_graphs=True, timed_library_products=timed_library_products)
 
 
 def plain_rows(folder, seqs, places, weights_as=torch.float32):

@@ -193,6 +193,30 @@ def test_many_decoding_rows_at_real_widths(shape_folders, name, dtype, graphs):
     assert bad is None, f"shape {name}, {dtype}: first wrong place (request, position, error) = {bad}"
 
 
+def test_recorded_steps_without_timed_products_give_the_same_bits_twice(shape_folders):
+    """Two runners made one after the other with ``timed_library_products`` off replay the same
+    steps (64 decoding rows beside portions, where the products are the library's) to logits
+    that are equal bit for bit: every product runs the library's first proposal, whatever a
+    runner before them has timed. With the timing on the same steps stay within the tolerance
+    of the plain model (the tests above) but need not give the same bits in another process."""
+    folder = shape_folders("1b")
+    seqs, steps = many_decoders(SHAPES["1b"]["vocab_size"], 64, seed=9, long_len=200,
+                                want_prompt_rows="last", lengths=(20, 60), portion=100)
+    pages = cuttings.max_live_tokens(steps, round_to=16) // 16
+    # a runner that times the shapes of its recorded steps comes first
+    replay_wanted(load_graph_runner(folder, torch.bfloat16, 16, pages, max_model_len=320, max_num_seqs=65),
+                  steps)
+    got = []
+    for _ in range(2):
+        runner = load_graph_runner(folder, torch.bfloat16, 16, pages, max_model_len=320, max_num_seqs=65,
+                                   timed_library_products=False)
+        got.append(replay_wanted(runner, steps))
+        assert runner.graphs.buckets and runner.portion_graphs.buckets, "no step was replayed"
+        del runner
+    for rid in got[0]:
+        assert torch.equal(got[0][rid], got[1][rid]), f"request {rid}: the two runs differ"
+
+
 @pytest.fixture(scope="module")
 def full_depth(tmp_path_factory, gpu_device):
     """All sixteen layers of the 1B shape, as the measurements run it."""

@@ -165,3 +165,40 @@ def test_cache_sizing_counts_the_fixed_state():
     with pytest.raises(RuntimeError, match="no memory left"):
         pages_that_fit(fixed + per_page - 1, per_page, fixed, 1000)
     assert pages_that_fit(fixed, 0, fixed, 1000) == 1            # a model without paged layers
+
+
+def test_decode_copies_are_left_out_when_they_would_not_leave_room_for_the_cache(capsys, monkeypatch):
+    """The second copies of the weights take what the matrices take once more, plus the largest
+    of them while it is built; they are made only if the cache's floor stays free."""
+    import torch
+    import pytriton_llama_amd  # noqa: F401
+    from pytriton_llama_amd.config import EngineConfig, build_model
+    from pytriton_llama_amd.engine import llm
+    from tiny_configs import TINY_B
+    assert llm.decode_copies_fit(100, 30, 200, 70) and not llm.decode_copies_fit(100, 30, 200, 71)
+    model = build_model(TINY_B)
+    model.dtype = torch.float32
+    assert model.decode_copy_bytes() == (0, 0)                    # the decode kernels copy bfloat16 only
+    model.dtype = torch.bfloat16
+    copies, largest = model.decode_copy_bytes()
+    H, I, V, L = 128, 320, 384, 3
+    per_layer = (4 + 2 * 1) * 32 * H + H * 4 * 32 + 3 * I * H
+    assert copies == 2 * (L * per_layer + 2 * V * H) and largest == 2 * max(V * H, I * H)
+    made = []
+    monkeypatch.setattr(model, "make_decode_copies", lambda: made.append(1) or 0)
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (copies + largest + 999, 10 ** 9))
+    assert not llm.make_decode_copies_if_room(model, "cuda:0", 1000) and not made
+    assert "decode_weight_copies=False" in capsys.readouterr().err
+    assert llm.make_decode_copies_if_room(model, "cuda:0", 999) and made == [1]
+    # what the cache must get at least, and what recorded steps are allowed
+    ec = EngineConfig(dtype="bfloat16", page_size=16, max_model_len=64, max_num_seqs=4, use_graphs=False)
+    per_page = 2 * L * 1 * 16 * 32 * 2
+    assert llm.cache_floor_bytes(model, ec) == 4 * per_page
+    ec.num_pages = 9
+    assert llm.cache_floor_bytes(model, ec) == 9 * per_page
+    ec.use_graphs = True
+    rows = (4 + 2) * 32 + H + 2 * I + H                                  # q|k|v, o, gate|up, down
+    assert model.widest_step_row_bytes() == 2 * rows * 2
+    pool = llm.graph_pool_bytes(model, ec)
+    assert pool == (2048 + 4) * 2 * rows * 2 + 5 * V * 4
+    assert llm.cache_floor_bytes(model, ec) == 9 * per_page + pool

@@ -161,6 +161,33 @@ def test_gemm_library(ops, out_dtype, mnk):
         ops.gemm_library(x.float(), w)
 
 
+def test_gemm_library_runs_the_first_proposal_unless_asked_for_the_timed_one(ops):
+    """A shape for which the timing keeps another proposal than the library's first on this
+    GPU (64 rows, depth 8,192): calls outside ``timed_library_products`` give the same bits
+    before and after the timing, the timed choice agrees with them within the rounding of
+    bfloat16 (proposals add in different orders), and the choice can be asked for."""
+    M, N, K = 64, 2048, 8192
+    torch.manual_seed(11)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    before = ops.gemm_library(x, w)
+    with ops.timed_library_products():
+        timed = ops.gemm_library(x, w)
+        again = ops.gemm_library(x, w)
+    after = ops.gemm_library(x, w)
+    assert torch.equal(before, after)
+    assert torch.equal(timed, again)
+    choice = ops.library_product_choice(M, N, K, K)
+    assert choice >= 0
+    assert ops.library_product_choice(M + 1, N, K, K) == -1               # never timed
+    want = (x.double() @ w.double().T).float()
+    ulp = 2.0 ** -7 * want.abs() + 1e-3 * float(want.abs().max())
+    assert bool(((timed.float() - before.float()).abs() <= ulp).all())
+    torch.testing.assert_close(timed.float(), want, atol=2e-2, rtol=2e-2)
+    with ops.timed_library_products(False):                               # a switch passed on as off
+        assert torch.equal(ops.gemm_library(x, w), before)
+
+
 def test_gemm_library_times_nothing_while_a_graph_is_recorded(ops):
     """Timing switched on while a HIP graph is recorded: nothing waits for the stream there (the
     recording would fail), every replay gives the product, and the call after the recording,
