@@ -23,7 +23,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 
-from ..parts.base import PagedKVSpec, StateSpec
+from ..parts.base import PagedSpec, StateSpec
 
 RELEASED = -1   # block-table entry of a page that was given back (left of the window)
 
@@ -71,7 +71,7 @@ class PagePool:
 
 @dataclass
 class PagedGroup:
-    spec: PagedKVSpec
+    spec: PagedSpec
     layers: List[int]                 # cache-layer ids stored in this group, in order
     page_size: int
     pool: PagePool
@@ -93,7 +93,7 @@ class StateGroup:
 class CacheManager:
     def __init__(self, cache_layers: Sequence[object], page_size: int, num_pages,
                  max_num_seqs: int):
-        """cache_layers: one PagedKVSpec / StateSpec / None per cache layer of the
+        """cache_layers: one PagedSpec / StateSpec / None per cache layer of the
         model. num_pages: an int (every paged group gets that many) or one int
         per paged group."""
         if page_size <= 0 or max_num_seqs <= 0:
@@ -109,7 +109,7 @@ class CacheManager:
                 self.layer_home.append(None)
                 continue
             if spec not in by_spec:
-                if isinstance(spec, PagedKVSpec):
+                if isinstance(spec, PagedSpec):
                     by_spec[spec] = ("paged", len(self.paged))
                     self.paged.append(PagedGroup(spec, [], self.page_size, None))
                 elif isinstance(spec, StateSpec):

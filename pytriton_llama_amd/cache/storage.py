@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import List, Optional
+from typing import Dict, List, Optional
 
 import torch
 
@@ -11,13 +11,20 @@ from .manager import CacheManager
 
 @dataclass
 class PagedLayerView:
-    """What a mixer sees of one paged cache layer."""
-    k: torch.Tensor            # [num_pages, Hkv, page_size, D]
-    v: torch.Tensor
+    """What a mixer sees of one paged cache layer: the layer's pool of every tensor its
+    cache spec names, [num_pages, *page shape] each, also as attributes (``.k``, ``.v`` for
+    keys and values in pages of [Hkv, page_size, D])."""
+    tensors: Dict[str, torch.Tensor]
     group: int                 # index into StepContext.groups
     page_size: int
     writable: bool
     kind: str = "paged"
+
+    def __getattr__(self, name):               # (reached only for names that are no field)
+        try:
+            return self.__dict__["tensors"][name]
+        except KeyError:
+            raise AttributeError(f"this cache layer keeps no tensor {name!r}") from None
 
 
 @dataclass
@@ -30,23 +37,26 @@ class StateLayerView:
     kind: str = "state"
 
 
+def _element_size(dtype: torch.dtype) -> int:
+    return torch.empty((), dtype=dtype).element_size()
+
+
 class CacheStorage:
-    """Page pools [layers, num_pages, Hkv, page_size, D] for keys and for values
-    per paged group (the reference keeps one [max_tokens, 2*Hkv, D] tensor per
-    layer, lite_llama/executor/mem_manager.py:166-168), and one
-    [layers, max_num_seqs + 1, *shape] tensor per state group (the last row is the padding
-    slot of the manager)."""
+    """Per paged group and per tensor of its spec a pool [layers, num_pages, *page shape]
+    (for keys and values [layers, num_pages, Hkv, page_size, D]; the reference keeps one
+    [max_tokens, 2*Hkv, D] tensor per layer, lite_llama/executor/mem_manager.py:166-168), and
+    one [layers, max_num_seqs + 1, *shape] tensor per state group (the last row is the
+    padding slot of the manager)."""
 
     def __init__(self, manager: CacheManager, dtype: torch.dtype, device):
         self.manager = manager
-        self.k_pools: List[torch.Tensor] = []
-        self.v_pools: List[torch.Tensor] = []
+        self.paged_pools: List[Dict[str, torch.Tensor]] = []
         self.state_pools: List[torch.Tensor] = []
         for g in manager.paged:
-            shape = (len(g.layers), g.pool.num_pages, g.spec.num_kv_heads, g.page_size,
-                     g.spec.head_dim)
-            self.k_pools.append(torch.zeros(shape, dtype=dtype, device=device))
-            self.v_pools.append(torch.zeros(shape, dtype=dtype, device=device))
+            self.paged_pools.append({
+                t.name: torch.zeros((len(g.layers), g.pool.num_pages) + t.page_shape(g.page_size),
+                                    dtype=t.dtype or dtype, device=device)
+                for t in g.spec.tensors})
         for g in manager.states:
             shape = (len(g.layers), manager.max_num_seqs + 1) + tuple(g.spec.shape)
             self.state_pools.append(torch.zeros(shape, dtype=g.spec.dtype or dtype, device=device))
@@ -59,7 +69,7 @@ class CacheStorage:
             return None
         kind, g, i = home
         if kind == "paged":
-            return PagedLayerView(self.k_pools[g][i], self.v_pools[g][i], g,
+            return PagedLayerView({name: pool[i] for name, pool in self.paged_pools[g].items()}, g,
                                   self.manager.page_size, writable)
         return StateLayerView(self.state_pools[g][i], g, writable)
 
@@ -74,7 +84,7 @@ class CacheStorage:
         number of pages)."""
         total = 0
         for g in manager.states:
-            size = torch.empty((), dtype=g.spec.dtype or dtype).element_size()
+            size = _element_size(g.spec.dtype or dtype)
             n = 1
             for d in g.spec.shape:
                 n *= int(d)
@@ -83,6 +93,12 @@ class CacheStorage:
 
     @staticmethod
     def bytes_per_page(manager: CacheManager, dtype: torch.dtype) -> int:
-        size = torch.empty((), dtype=dtype).element_size()
-        return sum(2 * len(g.layers) * g.spec.num_kv_heads * g.page_size * g.spec.head_dim * size
-                   for g in manager.paged)
+        """Bytes that one more page of every paged group takes (all layers, all tensors)."""
+        total = 0
+        for g in manager.paged:
+            for t in g.spec.tensors:
+                n = g.page_size
+                for d in t.shape:
+                    n *= int(d)
+                total += len(g.layers) * n * _element_size(t.dtype or dtype)
+        return total

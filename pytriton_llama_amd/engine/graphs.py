@@ -35,11 +35,10 @@ from __future__ import annotations
 
 from typing import Dict, List, Sequence
 
-import numpy as np
 import torch
 
 from .. import ops
-from .batch import GroupContext, StepContext, StepEntry, take_pages
+from .batch import SeqInput, StepEntry, StepLayout, StepSizes, take_pages
 
 
 def bucket_sizes(max_num_seqs: int) -> List[int]:
@@ -51,61 +50,29 @@ def bucket_sizes(max_num_seqs: int) -> List[int]:
     return out
 
 
-class _Bucket:
-    """Static buffers, context and captured graph for one padded batch size."""
+class _Recorded:
+    """A size class of steps: the layout with its static buffers (pinned on the host, and the
+    device copy a replay reads), the context over them with the host's numbers set to the most
+    the class can bring, and the captured graph."""
 
-    def __init__(self, size: int, manager, width: int, device):
-        self.size, self.width = size, width
-        B, G = size, len(manager.paged)
-        names = [("token_ids", B), ("positions", B), ("ctx_len", B), ("state_slots", B),
-                 ("q_start", B + 1), ("logit_rows", B), ("work_off", B)]
-        for g in range(G):
-            names += [(f"slots{g}", B), (f"table{g}", B * width)]
-        self.spans, n = {}, 0
-        for name, k in names:
-            self.spans[name] = (n, k)
-            n += k
-        self.host = torch.zeros(n, dtype=torch.int32).pin_memory()
-        self.np = self.host.numpy()
-        self.dev = torch.zeros(n, dtype=torch.int32, device=device)
-        a, k = self.spans["q_start"]
-        self.np[a:a + k] = np.arange(B + 1)
-        a, k = self.spans["logit_rows"]
-        self.np[a:a + k] = np.arange(B)
-        for g in range(G):
-            a, k = self.spans[f"slots{g}"]
-            self.np[a:a + k] = -1
-        self.table_np = [self.view_np(f"table{g}").reshape(B, width) for g in range(G)]
-        # per row: (the block table whose pages the row holds, how many of them). The table is
-        # kept by identity, not by the request's name: a request that ends and comes again
-        # under the same name (after a preemption, say) has a new table with other pages.
-        self.row_owner = [[None] * B for _ in range(G)]
-        empty = self.dev[:0]
-        # every sequence is one 16-row block at row 0: the work list of the vector-FMA
-        # attention kernel, which takes the head sizes the split-KV kernel does not
-        all16 = (self.view("logit_rows"), self.view("work_off"))
-        groups = [GroupContext(self.view(f"table{g}").view(B, width), self.view(f"slots{g}"))
-                  for g in range(G)]
-        self.ctx = StepContext(
-            token_ids=self.view("token_ids"), positions=self.view("positions"),
-            q_start=self.view("q_start"), ctx_len=self.view("ctx_len"),
-            state_slots=self.view("state_slots"), logit_rows=self.view("logit_rows"),
-            work={"all16": all16, "multi16": (empty, empty), "multi64": (empty, empty),
-                  "multi128": (empty, empty)},
-            groups=groups,
-            num_tokens=B, num_seqs=B, num_logit_rows=B, logit_rows_are_identity=True,
-            num_decode_seqs=B, q_lens=[1] * B, ctx_lens=[0] * B, max_q_len=1, max_ctx_len=0)
+    def __init__(self, manager, work_lists, device, sizes: StepSizes, max_model_len: int):
+        self.sizes = sizes
+        self.layout = StepLayout(manager, work_lists, device, sizes)
+        self.layout.dev = torch.zeros_like(self.layout.host, device=device)
+        B, m = sizes.decode_rows, sizes.multi_seqs
+        # the split of the decode attention and the blocks of a portion are fixed at the
+        # recording: planned for the longest context and the most rows
+        self.ctx = self.layout.context([1] * B + [sizes.multi_tokens] * m, [max_model_len] * (B + m),
+                                       logit_rows_are_identity=(m == 0))
         self.graph = None
         self.logits = None
-        self.copied = None                 # event: the last copy of ``host`` has been made
+        self.copied = None                 # event: the last copy of the pinned buffer has been made
 
-    def view(self, name):
-        a, k = self.spans[name]
-        return self.dev[a:a + k]
-
-    def view_np(self, name):
-        a, k = self.spans[name]
-        return self.np[a:a + k]
+    def wait_for_last_copy(self) -> None:
+        """Steps are launched ahead of the GPU: the pinned buffer is written again only when
+        its last copy to the device has been made."""
+        if self.copied is not None:
+            self.copied.synchronize()
 
 
 def capture_forward(model, storage, ctx, device, pool=None, timed_products: bool = True):
@@ -126,7 +93,10 @@ def capture_forward(model, storage, ctx, device, pool=None, timed_products: bool
     return graph, logits
 
 
-class DecodeGraphs:
+class _Graphs:
+    """What the two kinds of recorded steps share: refreshing the device copy of a layout and
+    recording a size class the first time a step falls into it."""
+
     def __init__(self, model, manager, storage, max_model_len: int, device, pool=None,
                  timed_products: bool = True):
         self.model, self.manager, self.storage = model, manager, storage
@@ -135,8 +105,37 @@ class DecodeGraphs:
         self.timed_products = timed_products
         self.max_model_len = int(max_model_len)
         self.width = -(-self.max_model_len // manager.page_size)
-        self.sizes = bucket_sizes(manager.max_num_seqs)
-        self.buckets: Dict[int, _Bucket] = {}
+        self.work_lists = tuple(model.work_lists())
+
+    def _replay(self, b: _Recorded, refresh) -> None:
+        """``refresh()`` brings the pinned buffer to the device; the graph is recorded first if
+        this is the first step of its size class."""
+        if b.graph is None:
+            # Recording runs the step once for real beforehand. Keys and values written twice
+            # are the same keys and values, but a mixer with state of its own would take the
+            # step twice: while recording, every sequence's state is the padding slot's, which
+            # starts from zero like a new request's.
+            slot_of = b.layout.np_of["state_slots"]
+            real = slot_of.copy()
+            slot_of[:] = self.manager.padding_slot
+            self.storage.clear_slot(self.manager.padding_slot)
+            refresh()
+            b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device, self.pool,
+                                                self.timed_products)     # waits for the device at its end
+            slot_of[:] = real
+            b.copied = torch.cuda.Event()
+        refresh()
+        b.copied.record()
+        b.graph.replay()
+
+
+class DecodeGraphs(_Graphs):
+    """Steps whose entries all bring one token, one graph per batch-size bucket."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.sizes = bucket_sizes(self.manager.max_num_seqs)
+        self.buckets: Dict[int, _Recorded] = {}
 
     def fits(self, entries: Sequence[StepEntry]) -> bool:
         if len(entries) > self.sizes[-1]:
@@ -148,78 +147,34 @@ class DecodeGraphs:
                 return False
         return True
 
-    def _bucket(self, n: int) -> _Bucket:
+    def _bucket(self, n: int) -> _Recorded:
         size = next(s for s in self.sizes if s >= n)
         b = self.buckets.get(size)
         if b is None:
-            b = self.buckets[size] = _Bucket(size, self.manager, self.width, self.device)
+            b = self.buckets[size] = _Recorded(self.manager, self.work_lists, self.device,
+                                               StepSizes(size, 0, 0, self.width, size), self.max_model_len)
         return b
-
-    def _capture(self, b: _Bucket) -> None:
-        # the split of the decode attention is fixed at capture: plan it for the longest context
-        b.ctx.ctx_lens = [self.max_model_len] * b.size
-        b.ctx.max_ctx_len = self.max_model_len
-        b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device, self.pool,
-                                            self.timed_products)
 
     def step(self, entries: Sequence[StepEntry], token_feed=None) -> torch.Tensor:
         """Logits [wanted, vocab] of a step whose entries all bring one token.
         ``token_feed``: an int32 device tensor with the entries' tokens, for a step that is
         launched before the host knows them (the entries then carry placeholders)."""
-        m = self.manager
-        starts = take_pages(entries, m, self.model.vocab_size)
+        starts = take_pages(entries, self.manager, self.model.vocab_size)
         n = len(entries)
         b = self._bucket(n)
-        # Steps are launched ahead of the GPU: the pinned buffer is written again only when
-        # its last copy to the device has been made.
-        if b.copied is not None:
-            b.copied.synchronize()
-        np_ = b.view_np
-        np_("token_ids")[:n] = [e.tokens[0] for e in entries]
-        np_("positions")[:n] = starts
-        ctx = np_("ctx_len")
-        ctx[:n] = starts
-        ctx[:n] += 1
-        ctx[n:] = 0
-        slot_of = np_("state_slots")
-        slot_of[:n] = [m.slot_of[e.request] for e in entries]
-        slot_of[n:] = m.padding_slot
-        P = m.page_size
-        for g, group in enumerate(m.paged):
-            slots = np_(f"slots{g}")
-            slots[n:] = -1
-            table_np, owner = b.table_np[g], b.row_owner[g]
-            for i, (e, pos) in enumerate(zip(entries, starts)):
-                table = group.tables[e.request]
-                slots[i] = table[pos // P] * P + pos % P
-                have = owner[i]
-                if have is not None and have[0] is table and have[1] <= len(table) \
-                        and group.spec.window is None:
-                    if have[1] < len(table):
-                        table_np[i, have[1]:len(table)] = table[have[1]:]
-                else:
-                    table_np[i, :len(table)] = table
-                owner[i] = (table, len(table))
+        b.wait_for_last_copy()
+        # every row's logits are computed (the rows wanted are picked below)
+        b.layout.fill([SeqInput(e.request, e.tokens[0], s) for e, s in zip(entries, starts)], (),
+                      range(b.sizes.decode_rows))
+
         def refresh():
             # one short kernel reads the pinned buffer and, for a step launched ahead, the
             # tokens the step before left on the device
-            ops.stage_step(b.dev, b.host, token_feed, b.spans["token_ids"][0], n)
-        if b.graph is None:
-            # Recording runs the step once for real beforehand. Keys and values written twice
-            # are the same keys and values, but a mixer with state of its own would take the
-            # step twice: while recording, every row's state is the padding slot's.
-            real = slot_of.copy()
-            slot_of[:] = m.padding_slot
-            refresh()
-            self._capture(b)                      # waits for the device at its end
-            slot_of[:] = real
-            b.copied = torch.cuda.Event()
-        refresh()
-        b.copied.record()
-        b.graph.replay()
+            ops.stage_step(b.layout.dev, b.layout.host, token_feed, b.layout.spans["token_ids"][0], n)
+        self._replay(b, refresh)
         logits = b.logits
         rows = [i for i, e in enumerate(entries) if e.want]
-        if len(rows) == n and n == b.size:
+        if len(rows) == n and n == b.sizes.decode_rows:
             return logits
         if len(rows) == n:
             return logits[:n]
@@ -233,85 +188,15 @@ PORTION_BUCKETS = (32, 64, 128, 256, 512) + tuple(range(640, 2049, 128))
 MAX_PORTION_GRAPHS = 48          # pairs of (decoding rows, portion size) kept; others run eagerly
 
 
-class _PortionBucket:
-    """Static buffers, context and captured graph for a step of ``rows`` single-token entries
-    (padded) followed by one entry of up to ``size`` tokens (padded)."""
-
-    def __init__(self, rows: int, size: int, manager, width: int, max_model_len: int, device):
-        from .batch import GENERIC_BLOCK_ROWS, MFMA_BIG_BLOCK_ROWS, MFMA_BLOCK_ROWS
-        self.rows, self.size = B, T = rows, size
-        G = len(manager.paged)
-        blocks = {"16": GENERIC_BLOCK_ROWS, "64": MFMA_BLOCK_ROWS, "128": MFMA_BIG_BLOCK_ROWS}
-        names = [("token_ids", B + T), ("positions", B + T), ("ctx_len", B + 1),
-                 ("state_slots", B + 1), ("q_start", B + 2), ("logit_rows", B + 1)]
-        for tag, r in blocks.items():
-            n = -(-T // r)
-            names += [("ws_" + tag, n), ("wo_" + tag, n)]
-        names += [("ws_all16", B + -(-T // GENERIC_BLOCK_ROWS)), ("wo_all16", B + -(-T // GENERIC_BLOCK_ROWS))]
-        for g in range(G):
-            names += [(f"slots{g}", B + T), (f"table{g}", (B + 1) * width)]
-        self.spans, n = {}, 0
-        for name, k in names:
-            self.spans[name] = (n, k)
-            n += k
-        self.host = torch.zeros(n, dtype=torch.int32).pin_memory()
-        self.np = self.host.numpy()
-        self.dev = torch.zeros(n, dtype=torch.int32, device=device)
-        # the portion is sequence B of the step; its query blocks, last rows first
-        for tag, r in blocks.items():
-            self.view_np("ws_" + tag)[:] = B
-            self.view_np("wo_" + tag)[:] = np.arange(0, T, r)[::-1]
-        # every sequence in 16-row blocks (the kernel that takes the other head sizes)
-        n16 = -(-T // GENERIC_BLOCK_ROWS)
-        self.view_np("ws_all16")[:n16] = B
-        self.view_np("wo_all16")[:n16] = np.arange(0, T, GENERIC_BLOCK_ROWS)[::-1]
-        self.view_np("ws_all16")[n16:] = np.arange(B)
-        self.view_np("wo_all16")[n16:] = 0
-        self.view_np("q_start")[:B + 1] = np.arange(B + 1)
-        self.view_np("logit_rows")[:B] = np.arange(B)
-        work = {tag: (self.view("ws_" + tag), self.view("wo_" + tag)) for tag in blocks}
-        work["all16"] = (self.view("ws_all16"), self.view("wo_all16"))
-        groups = [GroupContext(self.view(f"table{g}").view(B + 1, width), self.view(f"slots{g}"))
-                  for g in range(G)]
-        self.table_np = [self.view_np(f"table{g}").reshape(B + 1, width) for g in range(G)]
-        self.ctx = StepContext(
-            token_ids=self.view("token_ids"), positions=self.view("positions"),
-            q_start=self.view("q_start"), ctx_len=self.view("ctx_len"),
-            state_slots=self.view("state_slots"), logit_rows=self.view("logit_rows"),
-            work={"all16": work["all16"], "multi16": work["16"], "multi64": work["64"],
-                  "multi128": work["128"]},
-            groups=groups,
-            num_tokens=B + T, num_seqs=B + 1, num_logit_rows=B + 1, logit_rows_are_identity=False,
-            num_decode_seqs=B, q_lens=[1] * B + [T], ctx_lens=[max_model_len] * (B + 1),
-            max_q_len=T, max_ctx_len=max_model_len)
-        self.graph = None
-        self.logits = None
-        self.copied = None                 # event: the last copy of ``host`` has been made
-
-    def view(self, name):
-        a, k = self.spans[name]
-        return self.dev[a:a + k]
-
-    def view_np(self, name):
-        a, k = self.spans[name]
-        return self.np[a:a + k]
-
-
-class PortionGraphs:
+class PortionGraphs(_Graphs):
     """Steps of single-token entries (any number up to the largest decode bucket, also none)
     and exactly one entry of 2 to 2,048 tokens with at most one wanted place."""
 
-    def __init__(self, model, manager, storage, max_model_len: int, device, pool=None,
-                 timed_products: bool = True):
-        self.model, self.manager, self.storage = model, manager, storage
-        self.device = device
-        self.pool = pool
-        self.timed_products = timed_products
-        self.max_model_len = int(max_model_len)
-        self.width = -(-self.max_model_len // manager.page_size)
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
         self.sizes = list(PORTION_BUCKETS)
-        self.row_sizes = [0] + bucket_sizes(manager.max_num_seqs)
-        self.buckets: Dict[tuple, _PortionBucket] = {}
+        self.row_sizes = [0] + bucket_sizes(self.manager.max_num_seqs)
+        self.buckets: Dict[tuple, _Recorded] = {}
 
     def _split(self, entries):
         """(indices of the single-token entries, index of the portion) or None."""
@@ -347,67 +232,24 @@ class PortionGraphs:
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Logits [wanted, vocab] in the order of the entries."""
-        m = self.manager
         ones, portion = self._split(entries)
         tokens_of: list = []
-        starts = take_pages(entries, m, self.model.vocab_size, tokens_of)
-        e, toks, start = entries[portion], tokens_of[portion], starts[portion]
-        k, n = len(ones), len(toks)
-        key = (next(r for r in self.row_sizes if r >= k), next(t for t in self.sizes if t >= n))
+        starts = take_pages(entries, self.manager, self.model.vocab_size, tokens_of)
+        e, toks = entries[portion], tokens_of[portion]
+        key = (next(r for r in self.row_sizes if r >= len(ones)),
+               next(t for t in self.sizes if t >= len(toks)))
         b = self.buckets.get(key)
         if b is None:
-            b = self.buckets[key] = _PortionBucket(key[0], key[1], m, self.width,
-                                                   self.max_model_len, self.device)
-        B = b.rows
-        # Steps that nobody waits for (nothing wanted) let the host run ahead of the GPU: the
-        # pinned buffer is written again only when its last copy has been made.
-        if b.copied is not None:
-            b.copied.synchronize()
-        np_ = b.view_np
-        tok, pos, ctx = np_("token_ids"), np_("positions"), np_("ctx_len")
-        tok[:k] = [entries[i].tokens[0] for i in ones]
-        pos[:k] = [starts[i] for i in ones]
-        tok[k:B] = 0
-        pos[k:B] = 0
-        ctx[:k] = pos[:k] + 1
-        ctx[k:B] = 0                                     # padding rows: attention reads nothing
-        tok[B:B + n] = toks
-        tok[B + n:] = 0
-        pos[B:B + n] = np.arange(start, start + n)
-        pos[B + n:] = 0
-        ctx[B] = start + n
-        np_("q_start")[B + 1] = B + n
-        slot_of = np_("state_slots")
-        slot_of[:k] = [m.slot_of[entries[i].request] for i in ones]
-        slot_of[k:B] = m.padding_slot
-        slot_of[B] = m.slot_of[e.request]
-        np_("logit_rows")[B] = B + (e.want[0] if e.want else n - 1)
-        P = m.page_size
-        for g, group in enumerate(m.paged):
-            slots, table_np = np_(f"slots{g}"), b.table_np[g]
-            for j, i in enumerate(ones):
-                table = group.tables[entries[i].request]
-                slots[j] = table[starts[i] // P] * P + starts[i] % P
-                table_np[j, :len(table)] = table
-                table_np[j, len(table):] = -1
-            slots[k:B] = -1
-            slots[B:B + n] = m.slot_array(e.request, g, start, n)
-            slots[B + n:] = -1
-            table = group.tables[e.request]
-            table_np[B, :len(table)] = table
-            table_np[B, len(table):] = -1
-        if b.graph is None:
-            # (as for decode steps: no request's state is touched by the run that records)
-            real = slot_of.copy()
-            slot_of[:] = m.padding_slot
-            b.dev.copy_(b.host, non_blocking=True)
-            b.graph, b.logits = capture_forward(self.model, self.storage, b.ctx, self.device,
-                                                self.pool, self.timed_products)
-            slot_of[:] = real
-            b.copied = torch.cuda.Event()
-        b.dev.copy_(b.host, non_blocking=True)
-        b.copied.record()
-        b.graph.replay()
+            B, T = key
+            b = self.buckets[key] = _Recorded(self.manager, self.work_lists, self.device,
+                                              StepSizes(B, 1, T, self.width, B + 1), self.max_model_len)
+        B = b.sizes.decode_rows
+        b.wait_for_last_copy()
+        # the logits of every single-token row and of one row of the portion are computed
+        wanted_row = B + (e.want[0] if e.want else len(toks) - 1)
+        b.layout.fill([SeqInput(entries[i].request, int(tokens_of[i][0]), starts[i]) for i in ones],
+                      [SeqInput(e.request, toks, starts[portion])], list(range(B)) + [wanted_row])
+        self._replay(b, lambda: b.layout.dev.copy_(b.layout.host, non_blocking=True))
         # rows of the graph's logits in the caller's order of entries (a copy: the next replay
         # of this bucket overwrites the graph's own buffer)
         row_of = {i: j for j, i in enumerate(ones)}

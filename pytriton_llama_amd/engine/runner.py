@@ -69,7 +69,8 @@ class ModelRunner:
         elif self.portion_graphs is not None and self.portion_graphs.fits(entries):
             logits = self.portion_graphs.step(entries)
         else:
-            ctx, _ = build_context(entries, self.manager, self.device, self.model.vocab_size)
+            ctx, _ = build_context(entries, self.manager, self.device, self.model.vocab_size,
+                                   self.model.work_lists())
             logits = self.model.forward(ctx, self.storage)
         for e in entries:
             self.manager.release_behind_window(e.request)

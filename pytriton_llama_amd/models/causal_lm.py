@@ -84,6 +84,14 @@ class CausalLM:
         return sum(p.make_decode_copies() for p in [self.embedding, *self.blocks, self.final_norm, self.head]
                    if hasattr(p, "make_decode_copies"))
 
+    def work_lists(self) -> Tuple[Any, ...]:
+        """The work lists (parts.base.WorkList) that the blocks' parts want built for every step."""
+        lists: Tuple[Any, ...] = ()
+        for block in self.blocks:
+            if hasattr(block, "work_lists"):
+                lists += tuple(block.work_lists())
+        return tuple(dict.fromkeys(lists))
+
     def decode_copy_bytes(self) -> Tuple[int, int]:
         """(bytes the decode copies of all parts take at most, bytes of the largest of them):
         every matrix of the checkpoint once more in the engine dtype; nothing for an engine

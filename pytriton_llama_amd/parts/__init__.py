@@ -1,4 +1,5 @@
-from .base import (PART_KINDS, PART_REGISTRY, PagedKVSpec, ParamSource, Part, StateSpec, build_part,
+from .base import (PART_KINDS, PART_REGISTRY, PagedSpec, PagedTensor, ParamSource, Part, StateSpec, WorkList,
+                   build_part, paged_kv_spec,
                    place, register_part)
 from .linear import linear
 from .norm import RMSNorm

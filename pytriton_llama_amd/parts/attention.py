@@ -7,9 +7,18 @@ from typing import List, Optional
 import torch
 
 from .. import ops
-from .base import (PagedKVSpec, ParamSource, Part, PendingProduct, PendingScale, as_tensor, place,
-                   register_part)
+from .base import (ParamSource, Part, PendingProduct, PendingScale, WorkList, as_tensor,
+                   paged_kv_spec, place, register_part)
 from .linear import LINEAR_LIBRARIES, decode_copy, linear
+
+
+# How the attention kernels cut the query rows of a step: 16 rows a work item for the vector-FMA
+# kernel (over all sequences, or over those the split-KV decode kernel does not take), 64 or 128
+# for the matrix-core kernel for prompt portions.
+ALL_16 = WorkList(16)
+PORTIONS_16 = WorkList(16, after_decode=True)
+PORTIONS_64 = WorkList(64, after_decode=True)
+PORTIONS_128 = WorkList(128, after_decode=True)
 
 
 @register_part("mixer", "paged_attention")
@@ -54,8 +63,11 @@ class PagedAttention(Part):
             libs += tuple(position.kernel_libraries)
         self.kernel_libraries = tuple(dict.fromkeys(libs))
 
+    def work_lists(self):
+        return (ALL_16, PORTIONS_16, PORTIONS_64, PORTIONS_128)
+
     def cache_spec(self):
-        return PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
+        return paged_kv_spec(self.num_kv_heads, self.head_dim, self.window)
 
     @property
     def graph_capturable(self) -> bool:
@@ -166,13 +178,13 @@ class PagedAttention(Part):
         if (ops.attention_prefill_mfma_fits(q.dtype, self.num_kv_heads, D, cache.page_size)
                 and q.stride(0) % 8 == 0):
             rows, groups = ops.attention_prefill_mfma_plan(
-                q.device, self.num_heads, D, ctx.work["multi64"][0].numel(),
-                ctx.work["multi128"][0].numel())
-            ws, wo = ctx.work["multi128" if rows == 128 else "multi64"]
+                q.device, self.num_heads, D, ctx.work[PORTIONS_64][0].numel(),
+                ctx.work[PORTIONS_128][0].numel())
+            ws, wo = ctx.work[PORTIONS_128 if rows == 128 else PORTIONS_64]
             ops.attention_prefill_mfma(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
                                        group.block_table, ws, wo, self.scale, window, rows, groups)
         else:
-            ws, wo = ctx.work["multi16"] if n_dec else ctx.work["all16"]
+            ws, wo = ctx.work[PORTIONS_16 if n_dec else ALL_16]
             ops.attention_generic(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
                                   group.block_table, ws, wo, self.scale, window)
 

@@ -15,8 +15,9 @@ every part:
                             names relative to the prefix the model gives the part
     load(tensors, dtype, device)   take them (keyed by the same names); may fuse
 norm:            forward(x, residual) -> (y, new_residual)    residual may be None
-mixer:           cache_spec() -> PagedKVSpec | StateSpec | None
+mixer:           cache_spec() -> PagedSpec | StateSpec | None
                  forward(x, ctx, cache) -> y      x, y: [T, hidden]
+                 work_lists() -> WorkList, ...   (optional) how its kernels cut the query rows
 feed-forward:    forward(x) -> y
 position:        rotary_inv_freq() -> float32 [D/2] or None;  apply(q, k, positions) in place
 embedding:       forward(token_ids int32 [T]) -> [T, hidden]
@@ -45,8 +46,11 @@ between blocks) asks the classes for these flags and passes plain tensors to eve
 ``ctx`` is the StepContext of engine/batch.py: the flat batch (positions,
 q_start, ctx_len, per cache group its block table and slot mapping, the state
 slot of every sequence). ``cache`` is the view of the one cache layer the call
-was given: for a paged spec .k/.v pools of that layer, .group, .writable; for a
-state spec .state [max_num_seqs, *shape].
+was given: for a paged spec the pools of that layer by the names of the spec's
+tensors (.k, .v for keys and values; .tensors[name]), .group, .page_size, .writable;
+for a state spec .state [max_num_seqs + 1, *shape]. The last row of a state tensor is
+the padding slot: rows that pad a recorded step to its size class name it (several rows
+of a step may), so it holds arbitrary values that no request ever reads.
 """
 from __future__ import annotations
 
@@ -69,12 +73,57 @@ class ParamSource:
 
 
 @dataclass(frozen=True)
-class PagedKVSpec:
-    """Keys and values of every token, in pages; ``window``: only the last
-    ``window`` positions are ever read again, older pages can be given back."""
-    num_kv_heads: int
-    head_dim: int
+class PagedTensor:
+    """One tensor that a paged cache layer keeps for every token. ``shape`` is that of one
+    token; a page of the tensor has the shape shape[:token_axis] + (page_size,) +
+    shape[token_axis:], so that a kernel can have the tokens of a page where it reads them
+    best (keys and values: (kv heads, head size) with token_axis 1 gives pages of
+    [kv heads, page_size, head size])."""
+    name: str
+    shape: Tuple[int, ...]
+    token_axis: int = 0
+    dtype: Optional[torch.dtype] = None     # None: the engine dtype
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        if not 0 <= self.token_axis <= len(self.shape):
+            raise ValueError(f"paged tensor {self.name!r}: token_axis {self.token_axis} outside "
+                             f"its {len(self.shape)} dimensions")
+        return tuple(self.shape[:self.token_axis]) + (int(page_size),) + tuple(self.shape[self.token_axis:])
+
+
+@dataclass(frozen=True)
+class PagedSpec:
+    """What a mixer keeps for every token, in pages: any number of named tensors. ``window``:
+    only the last ``window`` positions are ever read again, older pages can be given back.
+    Cache layers with equal specs share a page pool and a block table per request."""
+    tensors: Tuple[PagedTensor, ...]
     window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a paged cache spec needs tensors with names of their own, got {names}")
+
+
+def paged_kv_spec(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> PagedSpec:
+    """Keys and values of every token: tensors "k" and "v", pages of [kv heads, page_size, head size]."""
+    shape = (int(num_kv_heads), int(head_dim))
+    return PagedSpec((PagedTensor("k", shape, 1), PagedTensor("v", shape, 1)), window)
+
+
+@dataclass(frozen=True)
+class WorkList:
+    """A list of (sequence, first query row) pairs that cuts the query rows of a step into
+    blocks of ``block_rows`` rows, one block a work item of a kernel, the blocks with the most
+    keys first. A part names the lists its kernels walk (``work_lists()``); the engine builds
+    them for every step, also for the padded steps it records as graphs, and hands them over
+    as ``ctx.work[WorkList(...)]`` = (sequence int32 [W], first row int32 [W]). In a recorded
+    step W is the most the step's size class can need, and items beyond the real ones are
+    empty: their first row is not below the rows their sequence brings.
+    ``after_decode``: only the sequences after the leading ones that bring a single token
+    (which a kernel specialised for decoding takes)."""
+    block_rows: int
+    after_decode: bool = False
 
 
 @dataclass(frozen=True)

@@ -27,6 +27,14 @@ class PreNormBlock(Part):
     def cache_spec(self):
         return self.mixer.cache_spec() if hasattr(self.mixer, "cache_spec") else None
 
+    def work_lists(self):
+        """The work lists its parts want (parts.base.WorkList)."""
+        lists = ()
+        for p in self.children().values():
+            if hasattr(p, "work_lists"):
+                lists += tuple(p.work_lists())
+        return tuple(dict.fromkeys(lists))
+
     can_defer_output = True
 
     @property

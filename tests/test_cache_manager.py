@@ -5,10 +5,10 @@ import random
 import pytest
 
 from pytriton_llama_amd.cache import RELEASED, CacheManager, OutOfPages, OutOfSlots, PagePool
-from pytriton_llama_amd.parts import PagedKVSpec, StateSpec
+from pytriton_llama_amd.parts import StateSpec, paged_kv_spec
 
-FULL = PagedKVSpec(2, 16)
-WIN = PagedKVSpec(2, 16, window=10)
+FULL = paged_kv_spec(2, 16)
+WIN = paged_kv_spec(2, 16, window=10)
 
 
 def test_nine_pages_like_the_reference_scenarios():
@@ -148,9 +148,9 @@ def test_cache_sizing_counts_the_fixed_state():
     import torch
     from pytriton_llama_amd.cache import CacheStorage
     from pytriton_llama_amd.engine.llm import pages_that_fit
-    from pytriton_llama_amd.parts import PagedKVSpec, StateSpec
-    layers = [PagedKVSpec(2, 16), StateSpec((1000,), torch.float32), StateSpec((1000,), torch.float32),
-              PagedKVSpec(2, 16), StateSpec((8, 8), None)]
+    from pytriton_llama_amd.parts import StateSpec, paged_kv_spec
+    layers = [paged_kv_spec(2, 16), StateSpec((1000,), torch.float32), StateSpec((1000,), torch.float32),
+              paged_kv_spec(2, 16), StateSpec((8, 8), None)]
     m = CacheManager(layers, 16, 4, 10)
     assert m.padding_slot == 10 and m.padding_slot not in m._free_slots
     per_page = CacheStorage.bytes_per_page(m, torch.bfloat16)

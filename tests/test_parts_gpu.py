@@ -149,7 +149,8 @@ def test_attention_part_alone(gpu_device, dtype):
         mgr.admit("r")
         ys = []
         for lo, hi in ((0, 20), (20, 37)):
-            ctx, _ = build_context([StepEntry("r", [0] * (hi - lo), [])], mgr, gpu_device)
+            ctx, _ = build_context([StepEntry("r", [0] * (hi - lo), [])], mgr, gpu_device,
+                                   work_lists=att.work_lists())
             ys.append(att.forward(x[lo:hi].cuda(), ctx, store.view(0)))
             mgr.release_behind_window("r")
         got = torch.cat(ys).float().cpu()
@@ -382,8 +383,12 @@ def test_toy_state_mixer_keeps_graphs_and_steps_launched_ahead(gpu_device):
         runner = ModelRunner(model, page_size=8, num_pages=40, max_num_seqs=4, max_model_len=64,
                              use_graphs=True)
         assert runner.graphs is not None and len(runner.manager.states) == 1
+        # the padding slot belongs to nobody and may hold anything: what the rows that pad a
+        # step read there and write back reaches no request
+        runner.storage.state_pools[0][:, runner.manager.padding_slot] = float("nan")
         from engine_helpers import replay_wanted
         got = replay_wanted(runner, steps)
+        assert all(bool(torch.isfinite(v).all()) for v in got.values())
         places = cuttings.wanted_places(steps)
         for rid in seqs:
             ref = want[rid][places[rid]]
@@ -404,6 +409,126 @@ def test_toy_state_mixer_keeps_graphs_and_steps_launched_ahead(gpu_device):
     for p, o in zip(prompts, outs["eager"]):
         ref = state_on_device_plain(model, p + o)
         assert o == [int(ref[len(p) - 1 + i].argmax()) for i in range(len(o))]
+
+
+CHUNKED = {"architectures": ["ToyStateLM"], "vocab_size": 75, "hidden_size": 48, "inner": 96,
+           "layers": ["chunked", "attention", "chunked"], "order": [0, 1, 2], "decay": 0.85,
+           "toy_norm": False, "toy_ffn": False, "heads": 3, "kv_heads": 1, "head_dim": 16,
+           "initializer_range": 0.25}
+
+
+def test_toy_mixer_gets_the_work_list_it_asks_for(gpu_device):
+    """A mixer defined here that walks blocks of 32 query rows (no kernel of the package cuts
+    rows so) names that list and finds it in every step: launched kernel by kernel (the list
+    has exactly the step's blocks), in recorded decode steps and in recorded steps with a
+    portion (the list has the size class's length and ends in empty items). All cuttings agree
+    with the plain whole-sequence result; a row left out of the list would stay zero."""
+    from pytriton_llama_amd.config import build_model
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.parts import WorkList
+    from pytriton_llama_amd.weights import load_random_weights
+    from engine_helpers import replay_wanted
+    model = build_model(copy.deepcopy(CHUNKED))
+    assert model.graph_capturable()
+    assert WorkList(32) in model.work_lists() and WorkList(64, after_decode=True) in model.work_lists()
+    load_random_weights(model, 5, torch.float32, gpu_device, norm_std=0.1)
+    g = torch.Generator().manual_seed(3)
+    seqs = {f"r{i}": torch.randint(0, 75, (n,), generator=g).tolist() for i, n in enumerate([70, 33, 101, 45])}
+    want = {rid: hybrid_plain(model, t) for rid, t in seqs.items()}
+    for steps in (cuttings.whole(seqs), cuttings.tail_decode(seqs, 32), cuttings.portions(seqs),
+                  cuttings.mixed(seqs, seed=5)):
+        runner = ModelRunner(model, page_size=8, num_pages=40, max_num_seqs=4)
+        got = replay(runner, steps, seqs)
+        for rid in seqs:
+            err = (got[rid] - want[rid]).abs().max() / float(want[rid].abs().max())
+            assert err < 2e-4, (rid, float(err))
+    only_portions = cuttings.portions(seqs, sizes=(40, 2, 33, 5, 64))      # (no step of single tokens)
+    only_portions[0]["step"] = "portions"
+    for steps in (cuttings.tail_decode(seqs, 12), only_portions, cuttings.mixed(seqs, seed=6)):
+        for st in steps:                         # one wanted place a portion: such steps are replayed
+            for e in st["entries"]:
+                e["want"] = e["want"][-1:]
+        runner = ModelRunner(model, page_size=8, num_pages=48, max_num_seqs=4, max_model_len=128,
+                             use_graphs=True)
+        got = replay_wanted(runner, steps)
+        places = cuttings.wanted_places(steps)
+        for rid in seqs:
+            ref = want[rid][places[rid]]
+            err = (got[rid] - ref).abs().max() / ref.abs().max()
+            assert err < 2e-4, (rid, float(err))
+        assert runner.portion_graphs.buckets and (runner.graphs.buckets or steps[0]["step"] == "portions"), \
+            "nothing was replayed"
+        # the recorded lists are longer than any step's own
+        some = next(iter(runner.portion_graphs.buckets.values()))
+        assert some.ctx.work[WorkList(32)][0].numel() == some.sizes.decode_rows + -(-some.sizes.multi_tokens // 32) + 1
+
+
+LATENT = {"architectures": ["ToyStateLM"], "vocab_size": 60, "hidden_size": 40, "inner": 64, "latent": 12,
+          "layers": ["latent", "attention", "latent"], "order": [0, 1, 2], "decay": 0.5,
+          "toy_norm": True, "toy_ffn": True, "heads": 2, "kv_heads": 2, "head_dim": 16,
+          "initializer_range": 0.3}
+
+
+def latent_plain(model, ids):
+    """Whole-sequence logits of the LATENT toy model, no cache, formulas spelt out here."""
+    ids = torch.as_tensor(ids)
+    S = len(ids)
+    h, residual = model.embedding.weight.float().cpu()[ids], None
+    for call in model.schedule:
+        b = model.blocks[call.block]
+        s = h if residual is None else h + residual
+        h, residual = s - s.mean(-1, keepdim=True), s
+        m = b.mixer
+        if hasattr(m, "latent"):
+            c = h @ m.wc.float().cpu().T
+            q = h @ m.wq.float().cpu().T
+            scores = (q @ c.T) / m.latent ** 0.5
+            scores = scores.masked_fill(torch.triu(torch.ones(S, S, dtype=torch.bool), diagonal=1), float("-inf"))
+            h = (torch.softmax(scores, dim=-1) @ c) @ m.wo.float().cpu().T
+        else:
+            qkv = h @ m.qkv.float().cpu().T
+            q = qkv[:, :m.q_size].view(S, m.num_heads, m.head_dim)
+            k = qkv[:, m.q_size:m.q_size + m.kv_size].view(S, m.num_kv_heads, m.head_dim)
+            v = qkv[:, m.q_size + m.kv_size:].view(S, m.num_kv_heads, m.head_dim)
+            cos, sin = plain_llama.rope_cos_sin(m.position.inv_freq_host, torch.arange(S))
+            o = plain_llama.causal_attention(plain_llama.apply_rope(q, cos, sin),
+                                             plain_llama.apply_rope(k, cos, sin), v, m.scale)
+            h = o.reshape(S, -1) @ m.o.float().cpu().T
+        s = h + residual
+        h, residual = s - s.mean(-1, keepdim=True), s
+        ff = b.feed_forward
+        h = torch.relu(h @ ff.w1.float().cpu().T) @ ff.w2.float().cpu().T
+    s = h + residual
+    return (s - s.mean(-1, keepdim=True)) @ model.head.weight.float().cpu().T
+
+
+def test_toy_mixer_with_one_paged_tensor_a_token(gpu_device):
+    """A mixer defined here whose paged memory is a single tensor a token (no keys and values)
+    is given pages, a block table and slots like attention: its cache spec names the tensor,
+    the manager forms a group of its own for its two layers beside the attention layer's, and
+    all cuttings (with so few pages that they are used again) agree with the plain result."""
+    from pytriton_llama_amd.config import build_model
+    from pytriton_llama_amd.engine.runner import ModelRunner
+    from pytriton_llama_amd.weights import load_random_weights
+    model = build_model(copy.deepcopy(LATENT))
+    load_random_weights(model, 11, torch.float32, gpu_device)
+    g = torch.Generator().manual_seed(2)
+    seqs = {f"r{i}": torch.randint(0, 60, (n,), generator=g).tolist() for i, n in enumerate([61, 38, 90, 47, 70])}
+    want = {rid: latent_plain(model, t) for rid, t in seqs.items()}
+    for steps in (cuttings.whole(seqs), cuttings.tail_decode(seqs, 32), cuttings.portions(seqs),
+                  cuttings.mixed(seqs, seed=7)):
+        pages = cuttings.max_live_tokens(steps, round_to=8) // 8
+        assert pages < sum(-(-len(t) // 8) for t in seqs.values()) or len(steps) == len(seqs)
+        runner = ModelRunner(model, page_size=8, num_pages=pages, max_num_seqs=4)
+        specs = [grp.spec for grp in runner.manager.paged]
+        assert [tuple(t.name for t in sp.tensors) for sp in specs] == [("latent",), ("k", "v")]
+        assert [len(grp.layers) for grp in runner.manager.paged] == [2, 1]
+        assert runner.storage.paged_pools[0]["latent"].shape == (2, pages, 8, 12)
+        got = replay(runner, steps, seqs)
+        for rid in seqs:
+            err = (got[rid] - want[rid]).abs().max() / float(want[rid].abs().max())
+            assert err < 2e-4, (rid, float(err))
+        assert all(grp.pool.num_free == pages for grp in runner.manager.paged)
 
 
 def test_parts_that_wait_for_the_device_are_never_recorded(gpu_device):

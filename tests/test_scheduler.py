@@ -15,7 +15,7 @@ from pytriton_llama_amd.engine.batch import StepEntry
 from pytriton_llama_amd.engine.request import Request, SamplingParams
 from pytriton_llama_amd.engine.runner import ModelRunner
 from pytriton_llama_amd.engine.scheduler import Scheduler
-from pytriton_llama_amd.parts import PagedKVSpec
+from pytriton_llama_amd.parts import paged_kv_spec
 from pytriton_llama_amd.weights import load_random_weights
 
 
@@ -43,7 +43,7 @@ def run(sched, manager, max_steps=10_000, log=None):
 
 
 def make(num_pages=64, page=4, seqs=8, budget=32, chunk=None, max_len=None):
-    m = CacheManager([PagedKVSpec(1, 16)], page, num_pages, seqs)
+    m = CacheManager([paged_kv_spec(1, 16)], page, num_pages, seqs)
     return m, Scheduler(m, seqs, budget, chunk, max_len, eos_token_ids=(999,))
 
 

@@ -7,7 +7,8 @@ import torch
 
 from pytriton_llama_amd.config.registry import register_model
 from pytriton_llama_amd.models import CausalLM, LayerCall
-from pytriton_llama_amd.parts import (ParamSource, Part, StateSpec, build_part, place, register_part)
+from pytriton_llama_amd.parts import (PagedSpec, PagedTensor, ParamSource, Part, StateSpec, WorkList,
+                                      build_part, place, register_part)
 
 
 @register_part("embedding", "toy_embedding")
@@ -113,6 +114,102 @@ class ToyDecayStateOnDevice(Part):
         if cache.writable:
             cache.state.index_copy_(0, slots, s)
         return y.to(x.dtype)
+
+
+@register_part("mixer", "toy_chunked_decay")
+class ToyChunkedDecay(Part):
+    """The recurrence of ToyDecayState, s_t = decay * s_{t-1} + x_t W^T, y_t = s_t, worked out
+    block by block: the part asks the engine for a list that cuts the rows of a step into
+    blocks of 32 (another tiling than any kernel of the package has) and computes every block
+    of the list on its own, from the state at the start of the step and all rows of the
+    sequence up to the block's. Rows that no item of the list covers would stay zero. Nothing
+    is read on the host, so its steps are recorded as graphs, where the list is as long as the
+    size class can need and ends in empty items."""
+    BLOCKS = WorkList(32)
+
+    def __init__(self, hidden_size, decay):
+        self.hidden_size, self.decay = hidden_size, decay
+
+    def work_lists(self):
+        return (self.BLOCKS,)
+
+    def cache_spec(self):
+        return StateSpec((self.hidden_size,), torch.float32)
+
+    def param_sources(self):
+        return [ParamSource("w", (self.hidden_size, self.hidden_size))]
+
+    def load(self, tensors, dtype, device):
+        self.w = place(tensors["w"], "matrix", dtype, device)
+
+    def forward(self, x, ctx, cache):
+        u = x.float() @ self.w.float().T                                 # [T, H]
+        T, n = u.shape[0], ctx.num_seqs
+        seq, off = (t.long() for t in ctx.work[self.BLOCKS])            # [W] each
+        q_start = ctx.q_start.long()
+        first, end = q_start[seq], q_start[seq + 1]
+        rows = (first + off)[:, None] + torch.arange(32, device=u.device)[None, :]       # [W, 32]
+        live = rows < end[:, None]                                       # an empty item: no row
+        t = torch.arange(T, device=u.device)
+        dist = rows[:, :, None] - t[None, None, :]                       # [W, 32, T]
+        counts = (t[None, None, :] >= first[:, None, None]) & (dist >= 0) & live[:, :, None]
+        weights = torch.where(counts, torch.pow(self.decay, dist.clamp(min=0).float()),
+                              torch.zeros((), device=u.device))
+        y_blocks = torch.einsum("wat,th->wah", weights, u)
+        s0 = cache.state.index_select(0, ctx.state_slots.long()[seq])   # the state the step starts from
+        since = (rows - first[:, None] + 1).clamp(min=0).float()
+        y_blocks = y_blocks + torch.pow(self.decay, since)[:, :, None] * s0[:, None, :]
+        y = torch.zeros((T + 1, u.shape[1]), dtype=torch.float32, device=u.device)
+        # rows without a sequence go to a row of their own behind the last, which is dropped
+        y.index_copy_(0, torch.where(live, rows, torch.full_like(rows, T)).flatten(), y_blocks.flatten(0, 1))
+        if cache.writable:
+            # a sequence's new state is its last row's (a place without rows names the padding
+            # slot and writes there what nobody reads)
+            last = (q_start[1:n + 1] - 1).clamp(min=0)
+            cache.state.index_copy_(0, ctx.state_slots.long()[:n], y.index_select(0, last))
+        return y[:T].to(x.dtype)
+
+
+@register_part("mixer", "toy_latent_memory")
+class ToyLatentMemory(Part):
+    """A mixer whose paged memory is one tensor a token, not keys and values: it keeps
+    c_t = x_t Wc^T (``latent`` numbers) of every token in pages and a token reads all of them
+    up to its own, y_t = (sum_s p_ts c_s) Wo^T with p_t = softmax_s((x_t Wq^T) . c_s / sqrt(latent))."""
+    graph_capturable = False         # forward reads the tables on the host
+
+    def __init__(self, hidden_size, latent):
+        self.hidden_size, self.latent = hidden_size, latent
+
+    def cache_spec(self):
+        return PagedSpec((PagedTensor("latent", (self.latent,)),))
+
+    def param_sources(self):
+        H, L = self.hidden_size, self.latent
+        return [ParamSource("wc", (L, H)), ParamSource("wq", (L, H)), ParamSource("wo", (H, L))]
+
+    def load(self, tensors, dtype, device):
+        self.wc, self.wq, self.wo = (place(tensors[n], "matrix", dtype, device) for n in ("wc", "wq", "wo"))
+
+    def forward(self, x, ctx, cache):
+        L, P = self.latent, cache.page_size
+        group = ctx.groups[cache.group]
+        pool = cache.latent                                              # [pages, page_size, latent]
+        assert pool.shape[1:] == (P, L) and set(cache.tensors) == {"latent"}
+        c = x.float() @ self.wc.float().T
+        q = x.float() @ self.wq.float().T
+        if cache.writable:
+            pool.view(-1, L).index_copy_(0, group.slots.long(), c.to(pool.dtype))
+        starts, lens, tables = ctx.q_start.tolist(), ctx.ctx_len.tolist(), group.block_table.tolist()
+        y = torch.empty_like(c)
+        for i in range(ctx.num_seqs):
+            n, rows = lens[i], q[starts[i]:starts[i + 1]]
+            pages = torch.tensor(tables[i][:-(-n // P)], device=x.device)
+            memory = pool.index_select(0, pages).reshape(-1, L)[:n].float()
+            position = torch.arange(n - rows.shape[0], n, device=x.device)
+            scores = rows @ memory.T / L ** 0.5
+            scores = scores.masked_fill(torch.arange(n, device=x.device)[None, :] > position[:, None], float("-inf"))
+            y[starts[i]:starts[i + 1]] = torch.softmax(scores, dim=-1) @ memory
+        return (y @ self.wo.float().T).to(x.dtype)
 
 
 @register_part("feed_forward", "toy_relu")
@@ -227,6 +324,10 @@ def build_toy(cfg: ToyConfig) -> CausalLM:
             mixer = build_part("mixer", "toy_decay_state", hidden_size=H, decay=cfg.decay)
         elif kind == "state_on_device":
             mixer = build_part("mixer", "toy_decay_state_on_device", hidden_size=H)
+        elif kind == "chunked":
+            mixer = build_part("mixer", "toy_chunked_decay", hidden_size=H, decay=cfg.decay)
+        elif kind == "latent":
+            mixer = build_part("mixer", "toy_latent_memory", hidden_size=H, latent=cfg.latent)
         else:
             if getattr(cfg, "toy_position", False):
                 pos = build_part("position", "toy_decay", head_dim=cfg.head_dim, strength=0.02)
