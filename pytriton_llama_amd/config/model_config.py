@@ -140,8 +140,9 @@ class LlamaConfig:
             rope_theta=float(d.get("rope_theta", 10000.0)),
             rope_scaling=RopeScaling.from_dict(d.get("rope_scaling")),
             # absent: tied, as the reference's LlamaConfig has it
-            # (lite_llama/models/model_config.py:37-104); a checkpoint that then brings a head of
-            # its own is refused by the loader rather than run with the embedding table
+            # (lite_llama/models/model_config.py:37-104), unless the checkpoint brings a head of
+            # its own: then the file decides (tie_word_embeddings_given tells the model builder
+            # that config.json was silent)
             tie_word_embeddings=bool(d.get("tie_word_embeddings", True)),
             tie_word_embeddings_given=d.get("tie_word_embeddings") is not None,
             max_position_embeddings=d.get("max_position_embeddings"),

@@ -338,18 +338,39 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
   }
 }
 
+// Compute units of the current device (256 on MI355X), asked for once a device: the launch
+// rules below were measured there and are stated in compute units, not as numbers of that chip.
+static int compute_units() {
+  constexpr int MAX_DEVICES = 64;
+  static int cached[MAX_DEVICES];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      n = 256;
+    }
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 template <int MT, int U, int ROWS>
 static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
                               long ldy, int out_dtype, hipStream_t stream,
                               const AddNormArgs* an = nullptr, bool blocked = false) {
   if (blocked && K % 32) return PTL_ERR_ARG;
   const int blocks = (N + ROWS - 1) / ROWS;
-  // enough waves to keep every SIMD of 256 CUs busy a few times over, each with
-  // at least 256 elements of K to stream
+  // enough waves to keep every SIMD of the chip busy a few times over (16 waves a compute
+  // unit), each with at least 256 elements of K to stream
   // (measured on MI355X: 4 waves a workgroup are best from N = 2048 to N = 128256 at
   // K = 2048, 8 to 16 at K = 8192)
   int waves = 1;
-  while (waves < 16 && (long)blocks * waves < 4096 && K / (waves * 2) >= 256) waves <<= 1;
+  while (waves < 16 && (long)blocks * waves < 16L * compute_units() && K / (waves * 2) >= 256) waves <<= 1;
   if (waves < 4 && K >= 1024) waves = 4;
   int k_per_wave = ((K + waves - 1) / waves + 31) / 32 * 32;
   const size_t lds = waves > 1 ? (size_t)waves * MT * 64 * 4 * sizeof(float) : 0;
@@ -379,8 +400,10 @@ static int launch_skinny_rows(void* y, const void* x, const void* w, int M, int 
   return ptl_launch_status();
 }
 
-// weight rows a workgroup of the skinny kernel owns
-static int skinny_rows(int N) { return (N + 15) / 16 <= 160 ? 8 : 16; }
+// weight rows a workgroup of the skinny kernel owns: 8 while 16-row tiles would leave more than
+// three compute units in eight without one (160 tiles on 256 compute units)
+static int few_tiles() { return compute_units() * 5 / 8; }
+static int skinny_rows(int N) { return (N + 15) / 16 <= few_tiles() ? 8 : 16; }
 
 template <int MT, int U>
 static int launch_skinny(void* y, const void* x, const void* w, int M, int N, int K, long ldx,
@@ -407,7 +430,8 @@ extern "C" int ptl_gemm_skinny_bf16(void* y, const void* x, const void* w, int w
   return launch_skinny<4, 2>(y, x, w, M, N, K, ldx, ldy, out_dtype, stream, nullptr, bl);
 }
 
-// How many partial sums a row gets from ptl_gemm_skinny_add_norm_bf16 with N columns.
+// How many partial sums a row gets from ptl_gemm_skinny_add_norm_bf16 with N columns (on the
+// current device: the tile height follows its number of compute units).
 extern "C" int ptl_gemm_skinny_partials(int N) {
   const int rows = skinny_rows(N);
   return (N + rows - 1) / rows;
@@ -631,7 +655,7 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
 
 static int pair_waves(int blocks, int K) {
   int waves = 1;
-  while (waves < 16 && (long)blocks * waves < 4096 && K / (waves * 2) >= 256) waves <<= 1;
+  while (waves < 16 && (long)blocks * waves < 16L * compute_units() && K / (waves * 2) >= 256) waves <<= 1;
   if (waves < 4 && K >= 1024) waves = 4;
   return waves;
 }
@@ -681,7 +705,7 @@ extern "C" int ptl_qkv_rope_store_bf16(void* q_out, long ldq, const void* x, con
     return PTL_ERR_ARG;
   const RowScaleArgs sc = {partials, n_partials, 1.0f / (float)K, eps};
   // few heads: 8-column tiles, so that twice as many workgroups share the weight stream
-  const bool small = (Hq + 2 * Hkv) * (D / 32) <= 160;
+  const bool small = (Hq + 2 * Hkv) * (D / 32) <= few_tiles();
   const int tiles = small ? D / 16 : D / 32;      // tiles in half a head
   const int blocks = (Hq + 2 * Hkv) * tiles;
   const int waves = pair_waves(blocks, K);

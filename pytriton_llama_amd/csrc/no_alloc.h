@@ -15,13 +15,20 @@
 //     nothing has to be cleared between calls, but two calls that overlap in time on one GPU
 //     (different streams, or different threads) race: keep them on one stream or order them
 //     with events.
-//   * The first call on a device looks the array's address up (hipGetSymbolAddress, with that
-//     device current) and keeps it; no call allocates or frees device or host memory.
+//   * The array's address on a device is looked up once (hipGetSymbolAddress, with that device
+//     current) and kept: by ptl_argmax_static_init for the current device, or by the first call
+//     of ptl_argmax_static for the device of its stream. The look-up is no work for a stream
+//     that is being captured: a call on a capturing stream whose device has not been looked up
+//     returns -2 and records nothing, so call ptl_argmax_static_init (or ptl_argmax_static once)
+//     before the capture begins. No call allocates or frees device or host memory.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #define PTL_ARGMAX_STATIC_MAX_PARTIALS 16384
+
+// Looks the array's address up for the current device (see above). Returns 0 or -2.
+extern "C" int ptl_argmax_static_init(void);
 
 // out [R] int32 (device), logits [R, V] float32 with row stride ``stride`` (device), host_out:
 // null, or pinned host memory [R] that receives the choices as well. Ties go to the lowest

@@ -111,13 +111,27 @@ static __device__ __align__(256) unsigned char argmax_scratch[PTL_ARGMAX_STATIC_
 static void* argmax_scratch_at[ARGMAX_STATIC_MAX_DEVICES];
 static std::mutex argmax_scratch_lock;
 
-static int argmax_scratch_of_current_device(void** base) {
-  int dev = -1;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ARGMAX_STATIC_MAX_DEVICES) return PTL_ERR_LAUNCH;
+// The array's address on device ``dev``, looked up the first time with that device current.
+// ``may_look_up`` false: only what is known already (a look-up may load the code object onto the
+// device, which is no work for a stream that is being captured).
+static int argmax_scratch_of(int dev, bool may_look_up, void** base) {
+  if (dev < 0 || dev >= ARGMAX_STATIC_MAX_DEVICES) return PTL_ERR_LAUNCH;
   std::lock_guard<std::mutex> hold(argmax_scratch_lock);
   if (argmax_scratch_at[dev] == nullptr) {
+    if (!may_look_up) return PTL_ERR_LAUNCH;
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess) {
+      (void)hipGetLastError();
+      return PTL_ERR_LAUNCH;
+    }
+    if (current != dev && hipSetDevice(dev) != hipSuccess) {
+      (void)hipGetLastError();
+      return PTL_ERR_LAUNCH;
+    }
     void* p = nullptr;
-    if (hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch)) != hipSuccess || p == nullptr) {
+    const hipError_t found = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch));
+    if (current != dev) (void)hipSetDevice(current);
+    if (found != hipSuccess || p == nullptr) {
       (void)hipGetLastError();
       return PTL_ERR_LAUNCH;
     }
@@ -127,14 +141,41 @@ static int argmax_scratch_of_current_device(void** base) {
   return PTL_OK;
 }
 
+// The device a stream belongs to (the current device for the null stream).
+static int device_of(hipStream_t stream) {
+  int dev = -1;
+  if (stream != nullptr && hipStreamGetDevice(stream, &dev) == hipSuccess) return dev;
+  (void)hipGetLastError();
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return -1;
+  }
+  return dev;
+}
+
+extern "C" int ptl_argmax_static_init(void) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return PTL_ERR_LAUNCH;
+  }
+  void* base = nullptr;
+  return argmax_scratch_of(dev, true, &base);
+}
+
 extern "C" int ptl_argmax_static(int32_t* out, const float* logits, int R, int V, long stride,
                                  int32_t* host_out, hipStream_t stream) {
   if (R <= 0) return PTL_OK;
   if (!out || !logits || V <= 0 || stride < V || R > 65535) return PTL_ERR_ARG;
   const long chunks = ((long)V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
   if ((long)R * chunks > PTL_ARGMAX_STATIC_MAX_PARTIALS) return PTL_ERR_ARG;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+    (void)hipGetLastError();
+    capturing = hipStreamCaptureStatusNone;
+  }
   void* base = nullptr;
-  const int rc = argmax_scratch_of_current_device(&base);
+  const int rc = argmax_scratch_of(device_of(stream), capturing == hipStreamCaptureStatusNone, &base);
   if (rc != PTL_OK) return rc;
   float* ws_val = reinterpret_cast<float*>(base);
   int32_t* ws_idx = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(base) +

@@ -93,3 +93,36 @@ def test_argmax_static_refuses_what_exceeds_its_array(gpu_device):
     assert lib.ptl_argmax_static(_ptr(out), _ptr(logits), 8, 16, ctypes.c_long(16), None, _stream()) == 0
     torch.cuda.synchronize()
     assert out.cpu().eq(0).all()                 # all equal: the lowest index
+
+
+def test_argmax_static_recorded_into_a_graph(gpu_device):
+    """For callers under graph capture: after ptl_argmax_static_init (the look-up of the
+    library's array is no work for a capturing stream) the call is recorded into a HIP graph and
+    replayed on two different inputs, with eager work in between; every replay gives what the
+    existing entry point gives."""
+    lib = _lib()
+    lib.ptl_argmax_static_init.restype = ctypes.c_int
+    assert lib.ptl_argmax_static_init() == 0
+    g = torch.Generator().manual_seed(8)
+    logits = torch.zeros((7, 50000), dtype=torch.float32, device=gpu_device)
+    out = torch.full((7,), -7, dtype=torch.int32, device=gpu_device)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert _static(lib, logits, out) == 0                  # (warm-up on the side stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = _static(lib, logits, out)
+    assert rc == 0
+    for seed in (1, 2, 3):
+        fresh = torch.randn((7, 50000), generator=g).to(gpu_device)
+        fresh[seed, 49999 - seed] = 30.0
+        logits.copy_(fresh)
+        out.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _existing(lib, logits)                          # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), want.cpu()) and int(out[seed]) == 49999 - seed
