@@ -415,8 +415,113 @@ def _fused_x_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
             and w.is_contiguous() and w.data_ptr() % 16 == 0 and w.shape[1] == x.shape[1])
 
 
-def gate_up_silu_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
-    return _fused_x_ok(x, w) and w.shape[0] % 32 == 0
+# Rows up to which the products of csrc/gemm_rows.hip take a decode step of more than 16 rows (they
+# work up to 128). Measured on MI355X at the 1B widths against the library's product followed by
+# the separate kernel (cold weights, microseconds at 32 / 64 / 128 rows): output projection + norm
+# 10.7 / 11.9 / 14.7 against 12.1 / 12.5 / 12.2; down projection + norm 16.7 / 18.0 / 22.0 against
+# 19.4 / 26.2 / 24.9; gate-up + SiLU-multiply 19.7 / 22.5 / 32.5 against 21.6 / 22.5 / 25.4; q|k|v +
+# rotation + cache write 11.2 / 14.8 / 18.7 against 13.7 / 14.2 / 17.3; the head of 128,256 columns
+# 105 / 112 / 204 against 129 / 137 / 150.
+ROWS_MAX = {"plain": 64, "add_norm": 64, "gate_up": 64, "qkv": 32}
+
+
+def _rows_x_ok(x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Tensor], use: str = "") -> bool:
+    """Whether the kernels for more than 16 rows take x with this weight (they read the blocked
+    copy) and, with ``use``, whether they are the faster way for that many rows."""
+    return (blocked is not None and x.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and x.dim() == 2 and FUSED_MAX_ROWS < x.shape[0] <= ROWS_MAX.get(use, 128) and x.shape[1] % 32 == 0
+            and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and w.dim() == 2 and w.shape[1] == x.shape[1])
+
+
+def _rows_weight(w: torch.Tensor, blocked: torch.Tensor, what: str):
+    N, K = w.shape
+    if (blocked.dtype != torch.bfloat16 or not blocked.is_cuda or not blocked.is_contiguous()
+            or tuple(blocked.shape) != (-(-N // 16), K // 32, 16, 32) or blocked.data_ptr() % 16):
+        raise KernelError(f"{what}: the blocked copy does not belong to a [{N}, {K}] bfloat16 matrix")
+    return _ptr(blocked)
+
+
+def gemm_rows_fits(x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Tensor]) -> bool:
+    """Whether ``gemm_rows`` takes the product and is the faster way for it: without slices of K
+    it gives every compute unit a workgroup only if the matrix has 64 rows for each (a head)."""
+    return _rows_x_ok(x, w, blocked, "plain") and w.shape[0] >= 64 * compute_units(x.device)
+
+
+def gemm_rows(x: torch.Tensor, w: torch.Tensor, blocked: torch.Tensor,
+              out_dtype: Optional[torch.dtype] = None, splits: int = 1) -> torch.Tensor:
+    """y = x @ w.T for 17 to 128 rows of bfloat16 x, streaming the blocked copy of w once (see
+    csrc/gemm_rows.hip). Output bfloat16 or float32 [M, N]; with ``splits`` > 1 the float32
+    partial sums [splits, M, N] over that many slices of K (for ``sum_add_rmsnorm``)."""
+    if not _rows_x_ok(x, w, blocked):
+        raise KernelError("gemm_rows: needs 17 to 128 rows of bfloat16 x with aligned rows, K a multiple "
+                          "of 32 and the blocked copy of w")
+    M, K = x.shape
+    N = w.shape[0]
+    out_dtype = out_dtype or torch.bfloat16
+    if out_dtype not in (torch.bfloat16, torch.float32) or (splits > 1 and out_dtype != torch.float32):
+        raise KernelError("gemm_rows: output is bfloat16 or float32, partial sums are float32")
+    y = torch.empty((splits, M, N) if splits > 1 else (M, N), dtype=out_dtype, device=x.device)
+    lib = library.load("gemm_rows")
+    _check(lib.ptl_rows_gemm_bf16(_ptr(y), _ptr(x), _rows_weight(w, blocked, "gemm_rows"), M, N, K,
+                                  ctypes.c_long(x.stride(0)), ctypes.c_long(N),
+                                  _F32 if out_dtype == torch.float32 else _BF16, int(splits),
+                                  _stream()), "gemm_rows")
+    return y
+
+
+def gemm_rows_splits(M: int, N: int, K: int) -> int:
+    """The slices of K that ``gemm_rows`` should leave partial sums of when a norm follows."""
+    return int(library.load("gemm_rows").ptl_rows_gemm_splits(int(M), int(N), int(K)))
+
+
+def sum_add_rmsnorm(partials: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,
+                    eps: float) -> torch.Tensor:
+    """y = rmsnorm(bfloat16(sum of partials) + residual) * weight for float32 partial sums
+    [splits, M, N] (or a float32 product [M, N]); ``residual`` (bfloat16 [M, N]) becomes the sum
+    in place. One kernel (csrc/gemm_rows.hip)."""
+    _need_gpu(partials, residual, weight)
+    if partials.dim() == 2:
+        partials = partials.unsqueeze(0)
+    S, M, N = partials.shape
+    if (partials.dtype != torch.float32 or not partials.is_contiguous() or residual.dtype != torch.bfloat16
+            or residual.shape != (M, N) or not residual.is_contiguous() or weight.dtype != torch.float32
+            or weight.shape != (N,) or not weight.is_contiguous() or N % 8 or N > 8192):
+        raise KernelError("sum_add_rmsnorm: needs contiguous float32 partial sums [S, M, N], a bfloat16 "
+                          "residual [M, N], a float32 weight [N], N a multiple of 8 up to 8192")
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=partials.device)
+    lib = library.load("gemm_rows")
+    _check(lib.ptl_rows_sum_add_rmsnorm(_ptr(y), _ptr(partials), S, _ptr(residual), _ptr(weight), M, N,
+                                        ctypes.c_float(eps), _stream()), "sum_add_rmsnorm")
+    return y
+
+
+def gemm_rows_add_rmsnorm_fits(x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Tensor],
+                               residual: torch.Tensor, norm_weight: torch.Tensor) -> bool:
+    N = w.shape[0]
+    return (_rows_x_ok(x, w, blocked, "add_norm") and residual.dtype == torch.bfloat16 and residual.is_cuda
+            and residual.shape == (x.shape[0], N) and residual.is_contiguous()
+            and norm_weight.dtype == torch.float32 and norm_weight.is_cuda and norm_weight.is_contiguous()
+            and norm_weight.numel() == N and N % 8 == 0 and N <= 8192)
+
+
+def gemm_rows_add_rmsnorm(x: torch.Tensor, w: torch.Tensor, blocked: torch.Tensor, residual: torch.Tensor,
+                          norm_weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """rmsnorm(x @ w.T + residual) * norm_weight for 17 to 128 rows, ``residual`` replaced by the
+    sum: the product as float32 partial sums over slices of K (so that a matrix with few rows
+    still gives every compute unit a workgroup), then one kernel that adds them up and
+    normalises whole rows."""
+    M, K = x.shape
+    partials = gemm_rows(x, w, blocked, torch.float32, splits=gemm_rows_splits(M, w.shape[0], K))
+    return sum_add_rmsnorm(partials, residual, norm_weight, eps)
+
+
+def gate_up_silu_fits(x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Tensor] = None) -> bool:
+    """Whether ``gate_up_silu`` is the way to go for x. ``blocked``: the blocked copy of w, which
+    the kernel for more than 16 rows reads."""
+    if _fused_x_ok(x, w):
+        return w.shape[0] % 32 == 0
+    return _rows_x_ok(x, w, blocked, "gate_up") and w.shape[0] % 64 == 0
 
 
 def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = None,
@@ -424,12 +529,20 @@ def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = N
     """silu(x Wg^T) * (x Wu^T) for w = [Wg; Wu] ([2I, K]) and at most 16 rows of
     bfloat16 x, in one kernel (see csrc/gemm.hip). ``scale``: the factor that the rows
     of x still lack; it is applied to both products."""
-    if not gate_up_silu_fits(x, w):
-        raise KernelError("gate_up_silu: needs bfloat16, at most 16 rows, K a multiple of 8, "
-                          "I a multiple of 16, aligned rows")
+    if not ((_fused_x_ok(x, w) and w.shape[0] % 32 == 0) or (_rows_x_ok(x, w, blocked) and w.shape[0] % 64 == 0)):
+        raise KernelError("gate_up_silu: needs bfloat16, K a multiple of 8, I a multiple of 16, aligned "
+                          "rows, at most 16 of them (up to 128 with the blocked copy of w, K and I "
+                          "multiples of 32)")
     M, K = x.shape
     I = w.shape[0] // 2
     out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+    if M > FUSED_MAX_ROWS:
+        if scale is not None:
+            raise KernelError("gate_up_silu: more than 16 rows come with their factor applied")
+        _check(library.load("gemm_rows").ptl_rows_gate_up_silu(
+            _ptr(out), _ptr(x), _rows_weight(w, blocked, "gate_up_silu"), M, I, K,
+            ctypes.c_long(x.stride(0)), _stream()), "gate_up_silu")
+        return out
     lib = library.load("gemm")
     pp, count, eps = scale.args(M, K, "gate_up_silu") if scale is not None else _NO_SCALE
     wp, wb = _weight_arg(w, blocked, M, "gate_up_silu")
@@ -440,8 +553,11 @@ def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = N
     return out
 
 
-def qkv_rope_store_fits(x: torch.Tensor, w: torch.Tensor, head_dim: int) -> bool:
-    return _fused_x_ok(x, w) and head_dim % 32 == 0
+def qkv_rope_store_fits(x: torch.Tensor, w: torch.Tensor, head_dim: int,
+                        blocked: Optional[torch.Tensor] = None) -> bool:
+    """Whether ``qkv_rope_store`` is the way to go for x. ``blocked``: the blocked copy of w, which
+    the kernel for more than 16 rows reads."""
+    return (_fused_x_ok(x, w) or _rows_x_ok(x, w, blocked, "qkv")) and head_dim % 32 == 0
 
 
 def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
@@ -453,9 +569,10 @@ def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
     into the cache pages at ``slots``; returns the rotated q [M, Hq, D]. At most 16
     rows of bfloat16 x, head sizes in steps of 32 (see csrc/gemm.hip). ``scale``: the
     factor that the rows of x still lack; it is applied to the products."""
-    if not qkv_rope_store_fits(x, w, head_dim):
-        raise KernelError("qkv_rope_store: needs bfloat16, at most 16 rows, K a multiple of 8, "
-                          "a head size in steps of 32, aligned rows")
+    if not ((_fused_x_ok(x, w) or _rows_x_ok(x, w, blocked)) and head_dim % 32 == 0):
+        raise KernelError("qkv_rope_store: needs bfloat16, K a multiple of 8, a head size in steps of "
+                          "32, aligned rows, at most 16 of them (up to 128 with the blocked copy of w "
+                          "and K a multiple of 32)")
     M, K = x.shape
     Hq, Hkv, D = num_heads, num_kv_heads, head_dim
     if w.shape[0] != (Hq + 2 * Hkv) * D:
@@ -477,6 +594,17 @@ def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
                 raise KernelError(f"qkv_rope_store: {name} must be contiguous bfloat16 "
                                   f"[pages, {Hkv}, {page_size}, {D}]")
     q = torch.empty((M, Hq, D), dtype=torch.bfloat16, device=x.device)
+    if M > FUSED_MAX_ROWS:
+        if scale is not None:
+            raise KernelError("qkv_rope_store: more than 16 rows come with their factor applied")
+        # the projection as float32 partial sums over slices of K (few rows of W: so that every
+        # compute unit gets a workgroup), then one kernel that adds them up, rotates and stores
+        partials = gemm_rows(x, w, blocked, torch.float32, splits=gemm_rows_splits(M, w.shape[0], K))
+        _check(library.load("gemm_rows").ptl_rows_sum_rope_store(
+            _ptr(q), ctypes.c_long(Hq * D), _ptr(partials), partials.shape[0] if partials.dim() == 3 else 1, M,
+            _ptr(positions), _ptr(inv_freq), _ptr(slots), _ptr(k_cache), _ptr(v_cache), Hq, Hkv, D,
+            int(page_size), _stream()), "qkv_rope_store")
+        return q
     lib = library.load("gemm")
     pp, count, eps = scale.args(M, K, "qkv_rope_store") if scale is not None else _NO_SCALE
     wp, wb = _weight_arg(w, blocked, M, "qkv_rope_store")

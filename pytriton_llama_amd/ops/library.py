@@ -26,7 +26,7 @@ HIPCC_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-shared", "-std=c++17"
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 KERNEL_LIBRARIES = ("embedding", "norm", "rope", "attention", "attention_prefill", "activation",
-                    "gemm", "blaslt", "sampling", "probe")
+                    "gemm", "gemm_rows", "blaslt", "sampling", "probe")
 # options of single sources. attention_prefill: no value there is a NaN unless an input is, and
 # without the promise every maximum of scores is preceded by instructions that quiet its inputs
 EXTRA_FLAGS = {"attention_prefill": ["-fno-honor-nans"]}

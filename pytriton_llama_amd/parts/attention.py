@@ -106,7 +106,7 @@ class PagedAttention(Part):
         if isinstance(x, PendingScale) and fused and ops.qkv_rope_store_fits(x.values, self.qkv, D):
             x, scale = x.values, x.scale
         x = as_tensor(x)
-        if fused and ops.qkv_rope_store_fits(x, self.qkv, D):
+        if fused and ops.qkv_rope_store_fits(x, self.qkv, D, self.qkv_blocked):
             # the few rows of a decode step: projection, rotation and cache write in one kernel
             q = ops.qkv_rope_store(x, self.qkv, ctx.positions, rotary,
                                    group.slots if cache.writable else None, cache.k, cache.v,
@@ -130,6 +130,8 @@ class PagedAttention(Part):
                        cache.page_size)
         out = torch.empty((T, Hq, D), dtype=x.dtype, device=x.device)
         self.attend(out, q, cache, ctx, group)
+        if defer_output:                    # (the norm that follows picks the kernels by the rows)
+            return PendingProduct(out.view(T, Hq * D), self.o, self.o_blocked)
         return linear(out.view(T, Hq * D), self.o, blocked=self.o_blocked)
 
     # ---- which kernel takes which sequences --------------------------------------

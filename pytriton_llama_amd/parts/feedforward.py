@@ -51,10 +51,13 @@ class SwiGLU(Part):
         if isinstance(x, PendingScale) and ops.gate_up_silu_fits(x.values, self.gate_up):
             x, scale = x.values, x.scale
         x = as_tensor(x)
-        if ops.gate_up_silu_fits(x, self.gate_up):
+        if ops.gate_up_silu_fits(x, self.gate_up, self.gate_up_blocked):
             # the few rows of a decode step: product and SiLU-multiply in one kernel
             a = ops.gate_up_silu(x, self.gate_up, scale, blocked=self.gate_up_blocked)
             if defer_output:
                 return PendingProduct(a, self.down, self.down_blocked)
             return linear(a, self.down, blocked=self.down_blocked)
-        return linear(ops.silu_mul(linear(x, self.gate_up)), self.down)
+        a = ops.silu_mul(linear(x, self.gate_up, blocked=self.gate_up_blocked))
+        if defer_output:                    # (the norm that follows picks the kernels by the rows)
+            return PendingProduct(a, self.down, self.down_blocked)
+        return linear(a, self.down, blocked=self.down_blocked)

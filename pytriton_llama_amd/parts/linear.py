@@ -16,7 +16,7 @@ import torch
 
 from .. import ops
 
-LINEAR_LIBRARIES = ("gemm", "blaslt")
+LINEAR_LIBRARIES = ("gemm", "gemm_rows", "blaslt")
 SKINNY_ROWS = 8          # rows up to which the skinny kernel takes a bfloat16 product
 SKINNY_ROWS_F32 = 16     # ... when float32 output is wanted (the head)
 
@@ -44,6 +44,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     # library up to 8 rows (and ahead for the vocabulary-sized head); beyond that the library
     if (M <= SKINNY_ROWS or (to_f32 and M <= SKINNY_ROWS_F32)) and ops.gemm_skinny_fits(x, w):
         return ops.gemm_skinny(x, w, out_dtype, blocked=blocked)
+    # some tens of rows (a large decoding batch): the kernel that streams the blocked copy with
+    # x staged through LDS, where measured faster than the library
+    if ops.gemm_rows_fits(x, w, blocked):
+        return ops.gemm_rows(x, w, blocked, out_dtype)
     if ops.gemm_library_fits(x, w):
         return ops.gemm_library(x, w, out_dtype, checked=True)
     if to_f32:

@@ -15,7 +15,7 @@ class RMSNorm(Part):
     sum returned as the new residual (lite_llama/kernels/skip_rmsnorm.py:94-181;
     call sites lite_llama/models/llama.py:149,160,219). Without a residual the
     input itself is the residual (:181)."""
-    kernel_libraries = ("norm", "gemm")
+    kernel_libraries = ("norm", "gemm", "gemm_rows")
     takes_pending_product = True
 
     def __init__(self, size: int, eps: float, weight_name: str = "weight"):
@@ -39,6 +39,12 @@ class RMSNorm(Part):
                 y, scale = ops.gemm_skinny_add_norm(x.x, x.w, residual, self.weight, self.eps,
                                                     blocked=x.blocked)
                 return PendingScale(y, scale), residual
+            # some tens of rows: the product as partial sums over slices of K, then one kernel
+            # that adds them up, adds the residual and normalises
+            if (residual is not None and x.blocked is not None
+                    and ops.gemm_rows_add_rmsnorm_fits(x.x, x.w, x.blocked, residual, self.weight)):
+                y = ops.gemm_rows_add_rmsnorm(x.x, x.w, x.blocked, residual, self.weight, self.eps)
+                return y, residual
         x = as_tensor(x)
         y = ops.add_rmsnorm(x, residual, self.weight, self.eps)
         return y, (x if residual is None else residual)

@@ -440,6 +440,121 @@ def test_decode_kernels_read_the_blocked_copy_of_a_weight(ops, dims):
     assert ops.blocked_weight(rnd(8, 40).to(torch.bfloat16).to(dev)) is None       # K no multiple of 32
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["to_bf16", "to_fp32"])
+@pytest.mark.parametrize("mnk", [(17, 64, 32), (24, 1000, 96), (33, 2048, 2080), (64, 130, 4096), (100, 3000, 160),
+                                 (128, 16400, 512), (5, 70, 64)])
+def test_gemm_rows(ops, out_dtype, mnk):
+    """The product for some tens of rows (x through LDS, the blocked copy of W streamed): widths
+    that are no multiple of a workgroup's 64 rows or of a tile's 16, depths that are no multiple
+    of a chunk, one and two tiles of W a wave, against a float64 product; and as partial sums
+    over slices of K, whose sum is the product."""
+    M, N, K = mnk
+    torch.manual_seed(21)
+    wide = torch.randn(M, K + 8, device="cuda").to(torch.bfloat16)
+    x = wide[:, :K]                                               # rows of a wider buffer
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    b = ops.blocked_weight(w)
+    want = (x.double() @ w.double().T).float()
+    t = dict(atol=1e-4, rtol=1e-4) if out_dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    y = ops.gemm_rows(x, w, b, out_dtype) if M > 16 else None
+    if M > 16:
+        assert y.dtype == out_dtype and y.shape == (M, N)
+        torch.testing.assert_close(y.float(), want, **t)
+        for splits in (2, 3, 8):
+            parts = ops.gemm_rows(x, w, b, torch.float32, splits=splits)
+            assert parts.shape == (splits, M, N)
+            torch.testing.assert_close(parts.sum(dim=0), want, atol=1e-4, rtol=1e-4)
+        with pytest.raises(ops.KernelError):
+            ops.gemm_rows(x, w, b, torch.bfloat16, splits=2)      # partial sums are float32
+        with pytest.raises(ops.KernelError):
+            ops.gemm_rows(x, w, torch.zeros_like(b)[1:], out_dtype)   # a copy of another matrix
+    else:
+        with pytest.raises(ops.KernelError):
+            ops.gemm_rows(x, w, b, out_dtype)                      # 16 rows and fewer: the other kernels
+
+
+@pytest.mark.parametrize("mnk", [(17, 64, 96), (40, 2048, 2048), (64, 2056, 320), (128, 4096, 8192)])
+def test_gemm_rows_add_rmsnorm(ops, mnk):
+    """Partial sums over slices of K, then one kernel that adds them up, adds the residual and
+    normalises whole rows: the residual it leaves and its output are those of the product
+    followed by add_rmsnorm, and of the plain formulas."""
+    M, N, K = mnk
+    torch.manual_seed(22)
+    eps = 1e-5
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    b = ops.blocked_weight(w)
+    res = torch.randn(M, N, device="cuda").to(torch.bfloat16)
+    nw = (1.0 + 0.2 * torch.randn(N, device="cuda")).float()
+    r1, r2 = res.clone(), res.clone()
+    partials = ops.gemm_rows(x, w, b, torch.float32, splits=ops.gemm_rows_splits(M, N, K))
+    got = ops.sum_add_rmsnorm(partials, r1, nw, eps)
+    want = ops.add_rmsnorm(ops.gemm_nt(x, w), r2, nw, eps)               # the separate kernels
+    torch.testing.assert_close(r1.float(), r2.float(), atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(got.float(), want.float(), atol=3e-2, rtol=2e-2)
+    h = (x.double() @ w.double().T).float().cpu() + res.float().cpu()
+    plain, plain_res = plain_llama.add_rms_norm(h, None, nw.cpu(), eps)
+    torch.testing.assert_close(got.float().cpu(), plain, atol=5e-2, rtol=3e-2)
+    torch.testing.assert_close(r1.float().cpu(), plain_res, atol=3e-2, rtol=2e-2)
+    # a float32 product of one piece is a partial sum of one slice
+    r3 = res.clone()
+    one = ops.sum_add_rmsnorm(ops.gemm_rows(x, w, b, torch.float32), r3, nw, eps)
+    torch.testing.assert_close(one.float(), got.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("mik", [(17, 64, 64), (33, 8192, 2048), (64, 352, 160), (128, 1024, 4096)])
+def test_gate_up_silu_for_tens_of_rows(ops, mik):
+    M, I, K = mik
+    torch.manual_seed(23)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(2 * I, K, device="cuda") / math.sqrt(K) * 2).to(torch.bfloat16)
+    got = ops.gate_up_silu(x, w, None, ops.blocked_weight(w))
+    gu = (x.double() @ w.double().T).float()
+    plain = plain_llama.silu(gu[:, :I]) * gu[:, I:]
+    torch.testing.assert_close(got.float(), plain, atol=3e-2, rtol=3e-2)
+    with pytest.raises(ops.KernelError):
+        ops.gate_up_silu(x, w)                                           # no blocked copy: not this many rows
+
+
+@pytest.mark.parametrize("dims", [(4, 2, 64, 16, 96, 20), (3, 1, 32, 4, 128, 33), (32, 8, 128, 16, 4096, 64),
+                                  (6, 3, 96, 8, 224, 128)])
+def test_qkv_rope_store_for_tens_of_rows(ops, dims):
+    """Partial sums of the projection, then one kernel that adds them up, rotates q and k and
+    writes k and v into their pages, against the plain formulas; rows whose slot is -1 store
+    nothing."""
+    Hq, Hkv, D, P, K, M = dims
+    torch.manual_seed(24)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = (torch.randn((Hq + 2 * Hkv) * D, K, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    positions = torch.randint(0, 100000, (M,), device="cuda").to(torch.int32)
+    positions[0] = 0
+    inv_freq = plain_llama.rope_inv_freq_default(500000.0, D).cuda()
+    pages = -(-M // P) + 2
+    slots = torch.randperm(pages * P, device="cuda")[:M].to(torch.int32)
+    slots[3] = -1
+    kc = torch.zeros(pages, Hkv, P, D, device="cuda", dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    q = ops.qkv_rope_store(x, w, positions, inv_freq, slots, kc, vc, Hq, Hkv, D, P, None, ops.blocked_weight(w))
+    full = (x.double() @ w.double().T).float().cpu()
+    cos, sin = plain_llama.rope_cos_sin(inv_freq.cpu(), positions.cpu())
+    want_q = plain_llama.apply_rope(full[:, :Hq * D].view(M, Hq, D), cos, sin)
+    torch.testing.assert_close(q.float().cpu(), want_q, atol=3e-2, rtol=3e-2)
+    want_k = plain_llama.apply_rope(full[:, Hq * D:(Hq + Hkv) * D].view(M, Hkv, D), cos, sin)
+    want_v = full[:, (Hq + Hkv) * D:].view(M, Hkv, D)
+    flat_k = kc.permute(0, 2, 1, 3).reshape(pages * P, Hkv, D).float().cpu()
+    flat_v = vc.permute(0, 2, 1, 3).reshape(pages * P, Hkv, D).float().cpu()
+    stored = torch.zeros(pages * P, dtype=torch.bool)
+    for m in range(M):
+        sl = int(slots[m])
+        if sl < 0:
+            continue
+        stored[sl] = True
+        torch.testing.assert_close(flat_k[sl], want_k[m], atol=3e-2, rtol=3e-2)
+        torch.testing.assert_close(flat_v[sl], want_v[m], atol=3e-2, rtol=3e-2)
+    assert bool((flat_k[~stored] == 0).all()) and bool((flat_v[~stored] == 0).all())
+    assert int(stored.sum()) == M - 1
+
+
 def _rope_reference(x, positions, inv_freq):
     cos, sin = plain_llama.rope_cos_sin(inv_freq, positions)
     return plain_llama.apply_rope(x, cos, sin)

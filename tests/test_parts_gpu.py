@@ -70,9 +70,37 @@ def test_pending_values_between_parts(gpu_device):
     assert isinstance(t, torch.Tensor) and torch.equal(r3, r_plain)
     torch.testing.assert_close(t.float(), n1.float(), atol=3e-2, rtol=2e-2)
     assert as_tensor(t) is t
-    # float32 and many rows never defer
+    # any number of rows is left to the norm, which picks the kernels by the rows: for 40 rows
+    # (no blocked copy of the weights here) the product and the norm as separate kernels
     many = torch.randn(40, H, device="cuda").to(torch.bfloat16)
-    assert isinstance(ff1.forward(many, defer_output=True), torch.Tensor)
+    res40 = torch.randn(40, H, device="cuda").to(torch.bfloat16)
+    p40 = ff1.forward(many, defer_output=True)
+    assert isinstance(p40, PendingProduct) and p40.shape == (40, H)
+    r_a, r_b = res40.clone(), res40.clone()
+    got40, r_a = run_norm(norm, p40, r_a, consumer=ff2)
+    want40, r_b = norm.forward(ff1.forward(many), r_b)
+    assert isinstance(got40, torch.Tensor) and torch.equal(got40, want40) and torch.equal(r_a, r_b)
+    # ... and with the blocked copies, for 17 to 64 rows, the product as partial sums and one
+    # kernel that adds them up and normalises
+    # (widths that are multiples of 32, which the blocked copies need)
+    H2, I2 = 128, 256
+    ff3 = build_part("feed_forward", "swiglu", hidden_size=H2, intermediate_size=I2)
+    ff3.load({"gate_proj.weight": 0.1 * torch.randn(I2, H2), "up_proj.weight": 0.1 * torch.randn(I2, H2),
+              "down_proj.weight": 0.1 * torch.randn(H2, I2)}, torch.bfloat16, gpu_device)
+    norm2 = build_part("norm", "rmsnorm", size=H2, eps=1e-5)
+    norm2.load({"weight": 1 + 0.2 * torch.randn(H2)}, torch.bfloat16, gpu_device)
+    many = torch.randn(40, H2, device="cuda").to(torch.bfloat16)
+    res40 = torch.randn(40, H2, device="cuda").to(torch.bfloat16)
+    r_b = res40.clone()
+    want40, r_b = norm2.forward(ff3.forward(many), r_b)
+    ff3.make_decode_copies()
+    p40 = ff3.forward(many, defer_output=True)
+    assert isinstance(p40, PendingProduct) and p40.blocked is not None
+    r_c = res40.clone()
+    got40b, r_c = run_norm(norm2, p40, r_c, consumer=ff3)
+    assert isinstance(got40b, torch.Tensor)
+    torch.testing.assert_close(got40b.float(), want40.float(), atol=3e-2, rtol=2e-2)
+    torch.testing.assert_close(r_c.float(), r_b.float(), atol=2e-2, rtol=2e-2)
 
 
 def test_rotary_part_alone(gpu_device):
