@@ -41,10 +41,7 @@ namespace {
 enum { MODE_PLAIN = 0, MODE_SILU = 1 };
 
 constexpr int TILES = 4;                   // tiles of 16 weight rows a workgroup owns: 64 rows
-#ifndef NB_X
-#define NB_X 3
-#endif
-constexpr int NB = NB_X;                   // chunks of x in LDS: one in use, the others on their way
+constexpr int NB = 3;                      // chunks of x in LDS: one in use, two on their way
 // Columns of a chunk (KC) and chunks of W a wave has under way (DEPTH) for 2, 4 and 8 tiles of
 // x, with one tile of W a wave: 8 KB of weights a wave in flight, chunks of x of at most 32 KB.
 // Measured at 64 rows and the 1B widths: 128 to 512 columns a chunk and 2 to 12 chunks under
@@ -95,11 +92,6 @@ gemm_rows_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t*
   const int k_lo = blockIdx.y * k_per_split;
   const int k_hi = min(K, k_lo + k_per_split);
   const int nchunks = (k_hi - k_lo + KC - 1) / KC;
-  // Workgroups take the chunks of their slice in different orders (a sum does not care): all
-  // tiles of W start at multiples of the same power of two, and workgroups that walked them in
-  // step would all be asking the same few memory channels at any moment.
-  const int rot = nchunks > 1 ? (blockIdx.x * 5 + blockIdx.y * 3) % nchunks : 0;
-  auto chunk_at = [&](int c) { const int p = c + rot; return p >= nchunks ? p - nchunks : p; };
 
   constexpr int WAVES = TILES / WT;              // waves that multiply, WT tiles of W each
   if (wave == WAVES) {
@@ -116,7 +108,7 @@ gemm_rows_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t*
       src[i] = min(row, M - 1) * (int)ldx + 8 * (place ^ (row & 15));
     }
     auto fetch = [&](int c) {
-      const int k = k_lo + chunk_at(c) * KC;
+      const int k = k_lo + c * KC;
       bf16_t* dst = xs + (size_t)(c % NB) * CHUNK;
 #pragma unroll
       for (int i = 0; i < XI; ++i) {
@@ -164,8 +156,7 @@ gemm_rows_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t*
     for (int t = 0; t < MT; ++t) acc[j][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   Frag8 ring[DEPTH][FRAGS][WT];
-  auto load_w = [&](Frag8 (&wf)[FRAGS][WT], int c_) {
-    const int c = chunk_at(c_);
+  auto load_w = [&](Frag8 (&wf)[FRAGS][WT], int c) {
 #pragma unroll
     for (int u = 0; u < FRAGS; ++u)
 #pragma unroll
