@@ -211,7 +211,10 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the 1B shape has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--points", default="1,64", help="other batch sizes to report, '' for none")
+    ap.add_argument("--points", default="1,16,32,64", help="other batch sizes to report, '' for none")
+    ap.add_argument("--long-context", type=int, default=8192, metavar="S",
+                    help="with the default run: one more point, batch 8 decoding behind prompts of S tokens "
+                         "(0: none)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-probes", action="store_true",
                     help="skip the two probes of the box (streaming read, MFMA loop)")
@@ -268,8 +271,8 @@ def main():
     log(f"model ready in {time.time() - t0:.1f}s")
     g = torch.Generator().manual_seed(1234)
 
-    def prompts(n):
-        return [torch.randint(0, cfg["vocab_size"], (S,), generator=g).tolist() for _ in range(n)]
+    def prompts(n, length=None):
+        return [torch.randint(0, cfg["vocab_size"], (length or S,), generator=g).tolist() for _ in range(n)]
 
     def sync():
         torch.cuda.synchronize()
@@ -302,13 +305,13 @@ def main():
         return 0
 
     # ---- decode ---------------------------------------------------------------------
-    def prefilled(batch, new_tokens, ends_there=False):
+    def prefilled(batch, new_tokens, ends_there=False, engine=engine, S=S, slack=slack):
         """``batch`` requests with their prompts in the cache and their first tokens sampled.
         ``ends_there``: every request ends with the token of decode step number ``new_tokens``
         from here, as the workload says (N new tokens each); the engine then launches no step
         ahead of the last one, so the timed steps are all that the GPU does inside the clock."""
         ids = [engine.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=new_tokens + slack - 4,
-                                                    ignore_eos=True)) for p in prompts(batch)]
+                                                    ignore_eos=True)) for p in prompts(batch, S)]
         while any(engine.requests[i].num_computed < S for i in ids):
             engine.step()                       # prompts go in, portion by portion
         if ends_there:
@@ -316,19 +319,21 @@ def main():
                 engine.requests[i].params.max_new_tokens = len(engine.requests[i].output) + new_tokens
         return ids
 
-    def drop(ids):
+    def drop(ids, engine=engine):
         for i in ids:
             engine.abort(i)                     # (nothing left to stop for a request that has ended)
         assert not engine.has_work
 
-    def decode_rate(batch, steps, warmup):
+    def decode_rate(batch, steps, warmup, engine=engine, S=S, slack=slack):
         """(tokens/s, seconds a step, mean context while timed, GB/s of what a step must read)"""
+        def prefilled_(b, n, ends_there=False):
+            return prefilled(b, n, ends_there, engine, S, slack)
         if warmup:
-            ids = prefilled(batch, warmup)      # a batch of the same shape takes the warm-up steps
+            ids = prefilled_(batch, warmup)     # a batch of the same shape takes the warm-up steps
             for _ in range(warmup):
                 engine.step()
-            drop(ids)
-        ids = prefilled(batch, steps, ends_there=True)
+            drop(ids, engine)
+        ids = prefilled_(batch, steps, ends_there=True)
         reqs = [engine.requests[i] for i in ids]
         first_ctx = [r.num_computed for r in reqs]
         sync()
@@ -341,7 +346,7 @@ def main():
         assert produced == batch * steps, (produced, batch, steps)
         assert all(r.finish_reason == "length" for r in reqs) and not engine.has_work
         ctx = [r.num_computed for r in reqs]
-        drop(ids)
+        drop(ids, engine)
         mean_ctx = (sum(first_ctx) + sum(ctx)) / (2.0 * len(ctx))
         bytes_step = nums["weight_bytes"] + batch * mean_ctx * nums["kv_bytes_per_token"]
         return batch * steps / dt, dt / steps, mean_ctx, bytes_step * steps / dt / 1e9
@@ -374,6 +379,27 @@ def main():
                 f"{made / dt:.0f} tok/s ({dt * 1e3:.0f} ms; the reference publishes 558 to 620 tok/s at batch 8)")
         except Exception as e:                                              # (never at the cost of the line)
             log(f"generate() call not measured: {e!r}")
+
+    # One point at a longer context: batch 8 decoding behind prompts of --long-context tokens, on a
+    # second engine that shares the weights (its recorded steps are planned for its own longest
+    # request, so the engine above keeps the plans of the workload it measures).
+    if args.points and args.long_context and args.long_context > S and not args.layers:
+        try:
+            model, S2, B2, K2, W2 = engine.model, args.long_context, 8, 32, 4
+            slack2 = B2 * -(-S2 // 2048) + 8
+            ec2 = EngineConfig(dtype=args.dtype, page_size=page,
+                               num_pages=-(-(S2 + K2 + slack2) // page) * B2 + 8, max_num_seqs=B2,
+                               max_num_batched_tokens=2048, prefill_chunk=2048,
+                               max_model_len=S2 + K2 + slack2, seed=0)
+            long_engine = Engine(model, ec2)
+            r, st, ctx2, gbs = decode_rate(B2, K2, W2, long_engine, S2, slack2)
+            points[f"decode_b{B2}_ctx{S2}"] = round(r, 1)
+            points[f"decode_b{B2}_ctx{S2}_ms_per_step"] = round(st * 1e3, 4)
+            points[f"decode_b{B2}_ctx{S2}_hbm_frac"] = round(gbs / PEAK_HBM_GBS, 4)
+            log(f"decode batch {B2} behind {S2}-token prompts: {r:.0f} tok/s, {st * 1e3:.3f} ms/step, {gbs:.0f} GB/s")
+            del long_engine
+        except Exception as e:                                              # (never at the cost of the line)
+            log(f"long-context point not measured: {e!r}")
 
     out = {
         "metric": f"decode tokens/s, {SHAPE_NAMES[args.shape]} shape, batch {args.batch}, {S}-token prompts",

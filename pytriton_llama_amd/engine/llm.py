@@ -109,7 +109,8 @@ class _Launched:
 
 
 class Engine:
-    """Model folder (or a config dict with ``random_seed``) -> generated tokens.
+    """Model folder (or a config dict with ``random_seed``, or a model that is built and loaded)
+    -> generated tokens.
 
         engine = Engine("/path/to/model", EngineConfig(dtype="bfloat16"))
         outs = engine.generate([[1, 2, 3]], SamplingParams(temperature=0, max_new_tokens=8))
@@ -121,7 +122,13 @@ class Engine:
         ec = self.config
         if torch.device(ec.device).type != "cuda":
             raise RuntimeError("the engine runs on a GPU only; there is no CPU path")
-        if isinstance(model, str):
+        if hasattr(model, "schedule") and hasattr(model, "blocks"):
+            # a model that is built and loaded (a CausalLM): another engine may share its weights
+            if model.dtype != ec.dtype or str(model.device) != str(torch.device(ec.device)):
+                raise ValueError(f"the model holds {model.dtype} on {model.device}, the engine is "
+                                 f"configured for {ec.dtype} on {ec.device}")
+            self.model = model
+        elif isinstance(model, str):
             cfg = read_config_json(model)
             self.model = build_model(cfg)
             if random_seed is None:
@@ -131,7 +138,7 @@ class Engine:
         else:
             self.model = build_model(model)
             load_random_weights(self.model, random_seed or 0, ec.dtype, ec.device, norm_std, weight_std)
-        if ec.decode_weight_copies:
+        if ec.decode_weight_copies and not self.model.has_decode_copies:
             make_decode_copies_if_room(self.model, ec.device, cache_floor_bytes(self.model, ec))
         num_pages = ec.num_pages if ec.num_pages is not None else pages_from_memory(self.model, ec)
         self.runner = ModelRunner(self.model, ec.page_size, num_pages, ec.max_num_seqs,

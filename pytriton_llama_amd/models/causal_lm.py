@@ -57,6 +57,7 @@ class CausalLM:
                                  f"there are {len(self.cache_layers)}")
         self.dtype: Optional[torch.dtype] = None
         self.device = None
+        self.has_decode_copies = False
 
     # ---- what the loader and the builder need -------------------------------
     def expected_tensors(self) -> Dict[str, Tuple[Part, ParamSource]]:
@@ -81,6 +82,7 @@ class CausalLM:
     def make_decode_copies(self) -> int:
         """Let every part build what it keeps beside its weights for faster decode steps;
         returns the bytes taken. After the weights are loaded."""
+        self.has_decode_copies = True
         return sum(p.make_decode_copies() for p in [self.embedding, *self.blocks, self.final_norm, self.head]
                    if hasattr(p, "make_decode_copies"))
 
