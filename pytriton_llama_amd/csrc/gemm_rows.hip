@@ -424,11 +424,23 @@ sum_add_rmsnorm_kernel(bf16_t* __restrict__ y, const float* __restrict__ partial
     const int ci = threadIdx.x + c * blockDim.x;
     if (ci < nchunk) {
       float p[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      for (int s = 0; s < splits; ++s) {
-        const float* at = partials + ((size_t)s * M + m) * N + (size_t)ci * 8;
-        const float4 a = *reinterpret_cast<const float4*>(at), b = *reinterpret_cast<const float4*>(at + 4);
-        p[0] += a.x; p[1] += a.y; p[2] += a.z; p[3] += a.w;
-        p[4] += b.x; p[5] += b.y; p[6] += b.z; p[7] += b.w;
+      // four slices' loads under way at a time (one after the other they would each cost a trip
+      // to L2), added in the order of the slices
+      for (int s0 = 0; s0 < splits; s0 += 4) {
+        float4 a[4], b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float* at = partials + ((size_t)min(s0 + j, splits - 1) * M + m) * N + (size_t)ci * 8;
+          a[j] = *reinterpret_cast<const float4*>(at);
+          b[j] = *reinterpret_cast<const float4*>(at + 4);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (s0 + j < splits) {
+            p[0] += a[j].x; p[1] += a[j].y; p[2] += a[j].z; p[3] += a[j].w;
+            p[4] += b[j].x; p[5] += b[j].y; p[6] += b[j].z; p[7] += b[j].w;
+          }
+        }
       }
       union { uint4 u; bf16_t e[8]; } r;
       r.u = *reinterpret_cast<const uint4*>(residual + (size_t)m * N + (size_t)ci * 8);
@@ -492,10 +504,17 @@ sum_rope_store_kernel(bf16_t* __restrict__ q_out, long ldq, const float* __restr
   const int head = p / half, j = p - head * half;
   const size_t width = (size_t)heads * D;
   float x1 = 0.f, x2 = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float* at = partials + ((size_t)s * M + m) * width + (size_t)head * D + j;
-    x1 += at[0];
-    x2 += at[half];
+  for (int s0 = 0; s0 < splits; s0 += 4) {       // (four slices' loads under way at a time)
+    float a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float* at = partials + ((size_t)min(s0 + i, splits - 1) * M + m) * width + (size_t)head * D + j;
+      a[i] = at[0];
+      b[i] = at[half];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (s0 + i < splits) { x1 += a[i]; x2 += b[i]; }
   }
   x1 = round_to<bf16_t>(x1);
   x2 = round_to<bf16_t>(x2);

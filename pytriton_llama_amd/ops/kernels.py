@@ -418,11 +418,11 @@ def _fused_x_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
 # Rows up to which the products of csrc/gemm_rows.hip take a decode step of more than 16 rows (they
 # work up to 128). Measured on MI355X at the 1B widths against the library's product followed by
 # the separate kernel (cold weights, microseconds at 32 / 64 / 128 rows): output projection + norm
-# 10.7 / 11.9 / 14.7 against 12.1 / 12.5 / 12.2; down projection + norm 16.7 / 18.0 / 22.0 against
-# 19.4 / 26.2 / 24.9; gate-up + SiLU-multiply 19.7 / 22.5 / 32.5 against 21.6 / 22.5 / 25.4; q|k|v +
-# rotation + cache write 11.2 / 14.8 / 18.7 against 13.7 / 14.2 / 17.3; the head of 128,256 columns
-# 105 / 112 / 204 against 129 / 137 / 150.
-ROWS_MAX = {"plain": 64, "add_norm": 64, "gate_up": 64, "qkv": 32}
+# 9.8 / 11.2 / 14.8 against 11.9 / 12.5 / 12.2; down projection + norm 15.8 / 17.2 / 21.7 against
+# 19.5 / 25.9 / 25.1; gate-up + SiLU-multiply 19.5 / 22.7 / 31.2 against 21.5 / 22.3 / 25.5; q|k|v +
+# rotation + cache write 10.0 / 13.7 / 18.5 against 13.7 / 14.1 / 17.1; the head of 128,256 columns
+# 101 / 112 / 206 against 131 / 137 / 150.
+ROWS_MAX = {"plain": 64, "add_norm": 64, "gate_up": 64, "qkv": 64}
 
 
 def _rows_x_ok(x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Tensor], use: str = "") -> bool:
