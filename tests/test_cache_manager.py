@@ -202,3 +202,37 @@ def test_decode_copies_are_left_out_when_they_would_not_leave_room_for_the_cache
     pool = llm.graph_pool_bytes(model, ec)
     assert pool == (2048 + 4) * 2 * rows * 2 + 5 * V * 4
     assert llm.cache_floor_bytes(model, ec) == 9 * per_page + pool
+
+
+def test_paged_specs_name_their_tensors():
+    """A paged layer keeps whatever tensors its spec names: keys and values, or one latent tensor
+    a token with a dtype of its own. Equal specs share a group, the storage makes a pool for
+    every tensor of a group, and a page costs what its tensors take."""
+    import torch
+    from pytriton_llama_amd.cache import CacheStorage
+    from pytriton_llama_amd.parts import PagedSpec, PagedTensor
+    latent = PagedSpec((PagedTensor("latent", (12,)), PagedTensor("gate", (3, 2), token_axis=1, dtype=torch.float32)))
+    same = PagedSpec((PagedTensor("latent", (12,)), PagedTensor("gate", (3, 2), token_axis=1, dtype=torch.float32)))
+    windowed = PagedSpec((PagedTensor("latent", (12,)),), window=7)
+    m = CacheManager([latent, FULL, same, windowed, None], page_size=8, num_pages=[5, 6, 4], max_num_seqs=2)
+    assert [len(g.layers) for g in m.paged] == [2, 1, 1]
+    assert m.layer_home == [("paged", 0, 0), ("paged", 1, 0), ("paged", 0, 1), ("paged", 2, 0), None]
+    s = CacheStorage(m, torch.bfloat16, "cpu")
+    assert s.paged_pools[0]["latent"].shape == (2, 5, 8, 12) and s.paged_pools[0]["latent"].dtype == torch.bfloat16
+    assert s.paged_pools[0]["gate"].shape == (2, 5, 3, 8, 2) and s.paged_pools[0]["gate"].dtype == torch.float32
+    assert set(s.paged_pools[1]) == {"k", "v"} and s.paged_pools[1]["k"].shape == (1, 6, 2, 8, 16)
+    per_page = 2 * 8 * (12 * 2 + 6 * 4) + 1 * 2 * 2 * 8 * 16 * 2 + 1 * 8 * 12 * 2
+    assert CacheStorage.bytes_per_page(m, torch.bfloat16) == per_page
+    view = s.view(2)
+    assert view.kind == "paged" and view.group == 0 and view.latent.shape == (5, 8, 12)
+    assert view.tensors["gate"].data_ptr() == s.paged_pools[0]["gate"][1].data_ptr()
+    with pytest.raises(AttributeError, match="keeps no tensor"):
+        view.k
+    kv = s.view(1)
+    assert kv.k.shape == (6, 2, 8, 16) and kv.v.shape == kv.k.shape
+    with pytest.raises(ValueError, match="names of their own"):
+        PagedSpec((PagedTensor("a", (2,)), PagedTensor("a", (3,))))
+    with pytest.raises(ValueError):
+        PagedTensor("x", (2,), token_axis=3).page_shape(4)
+    with pytest.raises(TypeError, match="unknown cache spec"):
+        CacheManager([("k", 2, 16)], 8, 4, 2)

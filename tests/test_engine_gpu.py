@@ -92,6 +92,32 @@ def test_cuttings_replayed_as_graphs(cases, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_a_replayed_portion_gives_the_logits_of_any_one_of_its_rows(cases, dtype):
+    """A replayed step with a portion computes the logits of one row of the portion: the row the
+    entry names, not only its last (first, a middle and the last row of portions of changing
+    size, alone and beside decoded tokens of another request), against the plain model."""
+    from engine_helpers import first_wrong_row, load_graph_runner, plain_rows, replay_wanted
+    folder, page, seqs, _ = cases["B"]
+    again = {r + "_again": t for r, t in seqs.items()}        # the same requests under other names
+    steps = cuttings.mixed(seqs, seed=11, max_live=3) + cuttings.portions(again, sizes=(9, 40, 2, 17))
+    for i, st in enumerate(steps):
+        st["step"] = i
+        for j, e in enumerate(st["entries"]):
+            n = len(e["tokens"])
+            e["want"] = [(0, n // 2, n - 1)[(i + j) % 3]] if n > 1 else [0]
+    assert any(e["want"] == [0] and len(e["tokens"]) > 2 for st in steps for e in st["entries"])
+    both = dict(seqs, **again)
+    places = cuttings.wanted_places(steps)
+    want = plain_rows(folder, both, places, dtype)
+    runner = load_graph_runner(folder, dtype, page, -(-cuttings.max_live_tokens(steps) // page),
+                               max_model_len=160, max_num_seqs=4)
+    got = replay_wanted(runner, steps)
+    bad = first_wrong_row(got, want, places, TOL[dtype])
+    assert bad is None, f"{dtype}: first wrong place (request, position, error) = {bad}"
+    assert runner.portion_graphs.buckets
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_first_tokens_of_a_sequence(cases, dtype):
     """Positions 0, 1, 2: one token whole, then one by one from an empty cache."""
     folder, page, seqs, want = cases["B"]
