@@ -33,10 +33,10 @@ silu_mul_bf16_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ gu
   const bf16_t* row0 = gu + ((size_t)t0 * 2 * I8 + c) * 8;
   const bf16_t* row1 = two ? row0 + (size_t)2 * I8 * 8 : row0;
   union { uint4 u; bf16_t e[8]; } g[2], u[2], o[2];
-  g[0].u = *reinterpret_cast<const uint4*>(row0);
-  u[0].u = *reinterpret_cast<const uint4*>(row0 + (size_t)I8 * 8);
-  g[1].u = *reinterpret_cast<const uint4*>(row1);
-  u[1].u = *reinterpret_cast<const uint4*>(row1 + (size_t)I8 * 8);
+  g[0].u = load_once(row0);
+  u[0].u = load_once(row0 + (size_t)I8 * 8);
+  g[1].u = load_once(row1);
+  u[1].u = load_once(row1 + (size_t)I8 * 8);
 #pragma unroll
   for (int r = 0; r < 2; ++r)
 #pragma unroll

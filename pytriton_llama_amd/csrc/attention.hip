@@ -589,15 +589,14 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, long out_stride, const bf16_t*
                        (uint32_t)(((kp & page_mask) * D + 8 * lg) * 2);
 #pragma unroll
       for (int kk = 0; kk < NDT; ++kk)
-        kf[u][kk].u = pk[u] >= 0 ? *reinterpret_cast<const uint4*>(kr + 64 * kk) : make_uint4(0, 0, 0, 0);
+        kf[u][kk].u = pk[u] >= 0 ? load_once(kr + 64 * kk) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < VCH; ++i) {
         const int vp = kc + 16 * u + vrow[i];
         vg[u][i] = make_uint4(0, 0, 0, 0);              // rows past the end read as zeros
         if (pv[u][i] >= 0)
-          vg[u][i] = *reinterpret_cast<const uint4*>(
-              v_head + (size_t)(uint32_t)pv[u][i] * page_bytes +
-              (uint32_t)(((vp & page_mask) * D + vcol[i]) * 2));
+          vg[u][i] = load_once(v_head + (size_t)(uint32_t)pv[u][i] * page_bytes +
+                               (uint32_t)(((vp & page_mask) * D + vcol[i]) * 2));
       }
     }
   };

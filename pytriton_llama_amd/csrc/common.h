@@ -28,6 +28,15 @@ __device__ __forceinline__ bf16_t float_to_bf16(float f) {
   return (bf16_t)(u >> 16);
 }
 
+// 16 bytes that a kernel reads once (weights, the cache of a decoding request, a product's result
+// on its way through an elementwise kernel): a load marked as not to be used again, so that it
+// does not displace what later kernels find in the caches.
+typedef unsigned int ptl_u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_once(const void* p) {
+  const ptl_u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const ptl_u32x4_t*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 template <typename T> __device__ __forceinline__ float to_float(T v);
 template <> __device__ __forceinline__ float to_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ float to_float<bf16_t>(bf16_t v) { return bf16_to_float(v); }

@@ -208,7 +208,7 @@ gemm_skinny_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const bool ok = k + 32 * u + 8 * lg < ke && wrow;
-      wf[u].u = ok ? *reinterpret_cast<const uint4*>(wp + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
+      wf[u].u = ok ? load_once(wp + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
     }
   };
   auto multiply = [&](GsFrag (&wf)[U], int k) {
@@ -521,8 +521,8 @@ gemm_pair_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x, const bf1
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const bool ok = k + 32 * u + 8 * lg < ke && wrow;
-      w1[u].u = ok ? *reinterpret_cast<const uint4*>(wp1 + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
-      w2[u].u = ok ? *reinterpret_cast<const uint4*>(wp2 + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
+      w1[u].u = ok ? load_once(wp1 + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
+      w2[u].u = ok ? load_once(wp2 + (k + 32 * u) * GS_KSTEP(BLOCKED)) : make_uint4(0, 0, 0, 0);
     }
   };
   auto load_x = [&](int k) {

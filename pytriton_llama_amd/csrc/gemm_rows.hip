@@ -161,7 +161,7 @@ gemm_rows_kernel(TY* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t*
     for (int u = 0; u < FRAGS; ++u)
 #pragma unroll
       for (int j = 0; j < WT; ++j)
-        wf[u][j].u = (k_lo + c * KC + 32 * u < k_hi) ? *reinterpret_cast<const uint4*>(wp[j] + (size_t)(c * FRAGS + u) * 512)
+        wf[u][j].u = (k_lo + c * KC + 32 * u < k_hi) ? load_once(wp[j] + (size_t)(c * FRAGS + u) * 512)
                                                      : make_uint4(0, 0, 0, 0);
   };
   // Every fragment of x that is read from LDS meets the WT tiles of W the wave owns. A chunk is

@@ -73,7 +73,7 @@ add_rmsnorm_bf16_vec_kernel(bf16_t* __restrict__ y, const bf16_t* __restrict__ x
     const int ci = threadIdx.x + c * blockDim.x;
     if (ci < nchunk) {
       union { uint4 u; bf16_t e[8]; } a, r;
-      a.u = *reinterpret_cast<const uint4*>(x + base + (size_t)ci * 8);
+      a.u = load_once(x + base + (size_t)ci * 8);
       if (has_residual) r.u = *reinterpret_cast<const uint4*>(residual + base + (size_t)ci * 8);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
