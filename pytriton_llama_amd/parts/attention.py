@@ -155,12 +155,13 @@ class PagedAttention(Part):
         if self.window:
             span = min(span, self.window)
         # measured on MI355X (256 compute units): the matrix-core kernel is best with about two
-        # workgroups a compute unit and without splits once the batch brings one for each; the
-        # other one with about four
+        # workgroups a compute unit, and without splits once the batch brings 1.75 for each
+        # (batch 56 with 8 kv heads; at batch 24 to 48 two splits are 2 to 3 % of a step faster
+        # than one); the other one with about four
         base = max(1, n_dec * groups)
         cus = ops.compute_units(device)
         if matrix_cores:
-            want = 1 if base >= cus else -(-2 * cus // base)
+            want = 1 if 4 * base >= 7 * cus else -(-2 * cus // base)
         else:
             want = -(-4 * cus // base)
         return max(1, min(want, -(-span // turn), 64))
