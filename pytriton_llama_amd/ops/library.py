@@ -14,6 +14,7 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
 import threading
 import time
 from typing import Dict, Iterable, List
@@ -115,16 +116,21 @@ def build(names: Iterable[str] = KERNEL_LIBRARIES, force: bool = False, verbose:
         tmp = final + f".tmp{os.getpid()}"
         if verbose:
             print(f"[pytriton_llama_amd] compiling {n}.hip for {ARCH} ...", file=sys.stderr, flush=True)
-        procs[n] = (subprocess.Popen(compile_command(n, tmp), stdout=subprocess.PIPE,
-                                     stderr=subprocess.STDOUT, text=True), tmp, final)
+        # the compiler's messages go to a file, not a pipe: nobody reads a pipe while the
+        # compiler runs, and one with many warnings would fill it and wait for ever
+        log = tempfile.TemporaryFile(mode="w+", encoding="utf-8", errors="replace")
+        procs[n] = (subprocess.Popen(compile_command(n, tmp), stdout=log, stderr=subprocess.STDOUT,
+                                     stdin=subprocess.DEVNULL), tmp, final, log)
     last = time.time()
     pending = dict(procs)
     errors = []
     while pending:
-        for n, (p, tmp, final) in list(pending.items()):
+        for n, (p, tmp, final, log) in list(pending.items()):
             if p.poll() is None:
                 continue
-            out = p.stdout.read()
+            log.seek(0)
+            out = log.read()
+            log.close()
             del pending[n]
             if p.returncode != 0:
                 errors.append(f"{n}.hip failed to compile:\n{out}")
