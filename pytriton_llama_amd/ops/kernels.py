@@ -753,17 +753,23 @@ def compute_units(device) -> int:
 
 
 def attention_prefill_mfma_plan(device: torch.device, num_heads: int, head_dim: int,
-                                blocks_of_64: int, blocks_of_128: int):
+                                blocks_of_64: int, blocks_of_128: int, max_keys: int = 0):
     """(block_rows, groups) for ``attention_prefill_mfma``, from sweeps on MI355X (one sequence
-    of 512 to 16,384 tokens, head sizes 64 and 128). With t = the workgroups a head can have
-    resident at once (three a compute unit up to head size 64, two above): 128-row blocks
-    (keys and values are staged half as often) once there are 1.25 t of them, 64-row blocks
-    before; a workgroup for every block while there are at most 2 t blocks (the longest start
-    first and the short ones fill in behind them), beyond that t workgroups that share the
-    sorted list as a snake, which evens out the causal triangle."""
+    of 512 to 16,384 tokens, and 2,048-token portions behind prefixes up to 14,336, head sizes
+    64 and 128). With t = the workgroups a head can have resident at once (three a compute unit
+    up to head size 64, two above): 128-row blocks (keys and values are staged half as often)
+    once there are 1.25 t of them, 64-row blocks before; at head sizes above 64 also from 0.5 t
+    on when some sequence has 4,096 keys or more (``max_keys``: the longest context of the
+    step, or a bound of it): a portion behind a long prefix has few blocks, all of them long
+    (at 32 heads of 128, 2,048 rows on 14,336 keys: 578 against 811 us; with no prefix the two
+    are level, at head size 64 they are level throughout). A workgroup for every block while
+    there are at most 2 t blocks (the longest start first and the short ones fill in behind
+    them), beyond that t workgroups that share the sorted list as a snake, which evens out the
+    causal triangle."""
     resident = compute_units(device) * (3 if head_dim <= 64 else 2)
     t = max(1, resident // num_heads)
-    rows, blocks = (128, blocks_of_128) if 4 * blocks_of_128 >= 5 * t else (64, blocks_of_64)
+    wide = 4 * blocks_of_128 >= 5 * t or (head_dim > 64 and max_keys >= 4096 and 2 * blocks_of_128 >= t)
+    rows, blocks = (128, blocks_of_128) if wide else (64, blocks_of_64)
     return rows, max(1, blocks if blocks <= 2 * t else t)
 
 

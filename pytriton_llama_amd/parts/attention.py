@@ -180,9 +180,10 @@ class PagedAttention(Part):
             return
         if (ops.attention_prefill_mfma_fits(q.dtype, self.num_kv_heads, D, cache.page_size)
                 and q.stride(0) % 8 == 0):
+            keys = max(ctx.ctx_lens[n_dec:])
             rows, groups = ops.attention_prefill_mfma_plan(
                 q.device, self.num_heads, D, ctx.work[PORTIONS_64][0].numel(),
-                ctx.work[PORTIONS_128][0].numel())
+                ctx.work[PORTIONS_128][0].numel(), min(keys, window) if window else keys)
             ws, wo = ctx.work[PORTIONS_128 if rows == 128 else PORTIONS_64]
             ops.attention_prefill_mfma(out, q, cache.k, cache.v, ctx.q_start, ctx.ctx_len,
                                        group.block_table, ws, wo, self.scale, window, rows, groups)

@@ -785,6 +785,14 @@ def test_attention_prefill_mfma_plan(ops):
     assert plan(2 * n128 - 2, n128 - 1)[0] == 64
     assert plan(8 * t, 4 * t) == (128, t)
     assert ops.attention_prefill_mfma_plan(dev, 4 * cus, 128, 1, 1) == (64, 1)
+    # head sizes above 64: 128-row blocks from 0.5 t blocks on when a context has 4,096 keys
+    t128 = max(1, 2 * cus // 32)
+    wide = lambda n128, keys: ops.attention_prefill_mfma_plan(dev, 32, 128, 2 * n128, n128, keys)
+    half = -(-t128 // 2)
+    assert wide(half, 4096) == (128, half) and wide(half, 4095)[0] == 64 and wide(half, 0)[0] == 64
+    if half > 1:
+        assert wide(half - 1, 16384)[0] == 64
+    assert plan(2 * half, half) == ops.attention_prefill_mfma_plan(dev, 32, 64, 2 * half, half, 16384)
 
 
 def test_attention_prefill_mfma_long(ops):
@@ -850,8 +858,9 @@ def test_attention_decode_long_contexts(ops, D, keys):
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("prefix,rows", [(14336, 2048), (8192, 8192)])
 def test_attention_prefill_mfma_long_prefix(ops, D, prefix, rows):
-    """A portion of 2,048 rows behind 14,336 keys in the cache (one workgroup a 64-row block by
-    the plan for 32 heads) and one of 8,192 rows behind 8,192 (128-row blocks, the list shared
+    """A portion of 2,048 rows behind 14,336 keys in the cache (one workgroup a block by the
+    plan for 32 heads: 64-row blocks at head size 64, 128-row blocks at head size 128, where
+    the long prefix decides) and one of 8,192 rows behind 8,192 (128-row blocks, the list shared
     by fewer workgroups than blocks), with the block size and workgroups that the plan gives
     and the work list the engine builds. Compared for the first, a middle and the last 128 rows;
     one query head a group points at one far key, the others are random with wide scores."""
@@ -865,9 +874,12 @@ def test_attention_prefill_mfma_long_prefix(ops, D, prefix, rows):
     q[:, 0::G] = 2.0
     _hot_keys(dk, kc, bt, P, 0, [0, 15, 16, 4095, 8192, prefix - 1, prefix, prefix + 5])
     n64, n128 = -(-rows // 64), -(-rows // 128)
-    block_rows, groups = ops.attention_prefill_mfma_plan(torch.device("cuda", 0), Hq, D, n64, n128)
+    block_rows, groups = ops.attention_prefill_mfma_plan(torch.device("cuda", 0), Hq, D, n64, n128, total)
     if rows == 8192:
         assert block_rows == 128 and groups < n128, "the case is meant to share the list"
+    elif torch.cuda.get_device_properties(0).multi_processor_count <= 256:
+        # few blocks, all of them long: 128 rows a block at head size 128, 64 at head size 64
+        assert block_rows == (128 if D > 64 else 64) and groups == (n128 if D > 64 else n64)
     ws, wo = work_items([rows], [total], 0, block_rows)
     dev = "cuda"
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
