@@ -1,4 +1,4 @@
-// The matrix products of a decode step with 17 to 128 rows (a batch of that many requests, one
+// The matrix products of a decode step with 9 to 128 rows (a batch of that many requests, one
 // token each), in bfloat16 on the matrix cores, with what follows a product done in its epilogue
 // or in one kernel behind it:
 //   ptl_rows_gemm_bf16        y = x W^T (bfloat16 or float32), or its float32 partial sums over
@@ -11,8 +11,8 @@
 // (lite_llama/models/llama.py:37-40,120, lite_llama/kernels/rope_emb.py, swiglu.py,
 // skip_rmsnorm.py).
 //
-// Such a step is bound by reading every weight once from HBM, like the steps of up to 16 rows
-// (gemm.hip), but its x is 2 to 8 MFMA tiles tall: a workgroup that owned 16 weight rows and
+// Such a step is bound by reading every weight once from HBM, like the steps of fewer rows
+// (gemm.hip), but its x is up to 8 MFMA tiles tall: a workgroup that owned 16 weight rows and
 // fetched its x from L2 would read 4 to 8 times more of x than of W, in half cache lines, and
 // the chip's L2 would be the bound (measured: 1.0 to 1.5 TB/s of weights). So here
 //   * a workgroup has four waves that multiply, each owning one tile of 16 weight rows and all
@@ -42,11 +42,12 @@ enum { MODE_PLAIN = 0, MODE_SILU = 1 };
 
 constexpr int TILES = 4;                   // tiles of 16 weight rows a workgroup owns: 64 rows
 constexpr int NB = 3;                      // chunks of x in LDS: one in use, two on their way
-// Columns of a chunk (KC) and chunks of W a wave has under way (DEPTH) for 2, 4 and 8 tiles of
+// Columns of a chunk (KC) and chunks of W a wave has under way (DEPTH) for 1, 2, 4 and 8 tiles of
 // x, with one tile of W a wave: 8 KB of weights a wave in flight, chunks of x of at most 32 KB.
 // Measured at 64 rows and the 1B widths: 128 to 512 columns a chunk and 2 to 12 chunks under
 // way differ by a few per cent. With two tiles a wave: 128 columns, 4 chunks (the head of
 // vocabulary size: 112 us against 137 with 256 and 2).
+constexpr int KC_1 = 256, DEPTH_1 = 2;
 constexpr int KC_2 = 256, DEPTH_2 = 2;
 constexpr int KC_4 = 256, DEPTH_4 = 2;
 constexpr int KC_8 = 128, DEPTH_8 = 4;
@@ -340,7 +341,7 @@ bool bad_common(int M, int K, long ldx) {
   return M <= 0 || M > 128 || K <= 0 || K % 32 || ldx % 8 || ldx < K;
 }
 
-int m_tiles(int M) { return M <= 32 ? 2 : M <= 64 ? 4 : 8; }
+int m_tiles(int M) { return M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8; }
 
 // The slices of K that a product should be cut into when the caller can take partial sums:
 // doubled while the workgroups are fewer than the compute units and a slice keeps at least 256
@@ -361,7 +362,7 @@ extern "C" int ptl_rows_gemm_splits(int M, int N, int K) {
 
 // y [splits, M, N] = x [M, K] W^T over ``splits`` slices of K (1: the product itself), W given
 // as its blocked copy (rows padded to a multiple of 16). out_dtype: bfloat16 (splits = 1 only)
-// or float32. 17..128 rows are what it is made for; fewer work too. splits: what
+// or float32. 9..128 rows are what it is made for; fewer work too. splits: what
 // ptl_rows_gemm_splits says, or 1.
 extern "C" int ptl_rows_gemm_bf16(void* y, const void* x, const void* w_blocked, int M, int N, int K,
                                   long ldx, long ldy, int out_dtype, int splits, hipStream_t stream) {
@@ -380,6 +381,7 @@ extern "C" int ptl_rows_gemm_bf16(void* y, const void* x, const void* w_blocked,
 #define BY_TYPE(MT, KC, DEPTH, WT) (out_dtype == PTL_DTYPE_F32 ? GO(MT, KC, DEPTH, WT, float) : GO(MT, KC, DEPTH, WT, bf16_t))
 #define BY_WT(MT, KC, DEPTH) (two ? BY_TYPE(MT, 128, 4, 2) : BY_TYPE(MT, KC, DEPTH, 1))
   switch (m_tiles(M)) {
+    case 1: return BY_WT(1, KC_1, DEPTH_1);
     case 2: return BY_WT(2, KC_2, DEPTH_2);
     case 4: return BY_WT(4, KC_4, DEPTH_4);
     default: return BY_WT(8, KC_8, DEPTH_8);
@@ -398,6 +400,7 @@ extern "C" int ptl_rows_gate_up_silu(void* out, const void* x, const void* w_blo
   const int blocks = I / 32;
 #define GO(MT, KC, DEPTH) launch<MT, KC, DEPTH, 1, MODE_SILU, bf16_t>(out, x, w_blocked, M, I, 2 * I, K, ldx, I, blocks, 1, I, stream)
   switch (m_tiles(M)) {
+    case 1: return GO(1, KC_1, DEPTH_1);
     case 2: return GO(2, KC_2, DEPTH_2);
     case 4: return GO(4, KC_4, DEPTH_4);
     default: return GO(8, KC_8, DEPTH_8);

@@ -415,21 +415,25 @@ def _fused_x_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
             and w.is_contiguous() and w.data_ptr() % 16 == 0 and w.shape[1] == x.shape[1])
 
 
-# Rows up to which the products of csrc/gemm_rows.hip take a decode step of more than 16 rows (they
+# Rows from which, and up to which, the products of csrc/gemm_rows.hip take a decode step (they
 # work up to 128). Measured on MI355X at the 1B widths against the library's product followed by
 # the separate kernel (cold weights, microseconds at 32 / 64 / 128 rows): output projection + norm
 # 9.8 / 11.2 / 14.8 against 11.9 / 12.5 / 12.2; down projection + norm 15.8 / 17.2 / 21.7 against
 # 19.5 / 25.9 / 25.1; gate-up + SiLU-multiply 19.5 / 22.7 / 31.2 against 21.5 / 22.3 / 25.5; q|k|v +
 # rotation + cache write 10.0 / 13.7 / 18.5 against 13.7 / 14.1 / 17.1; the head of 128,256 columns
-# 101 / 112 / 206 against 131 / 137 / 150.
+# 101 / 112 / 206 against 131 / 137 / 150. Against the fused kernels for at most 16 rows, whole
+# decode steps of 16 rows: 1.287 -> 1.243 ms at the 1B widths, 4.73 -> 4.58 ms at the 8B widths,
+# 3.04 -> 3.07 ms at the 3B widths (product by product the faster one depends on the shape): from
+# 9 rows on a step takes these kernels, where they fit.
+ROWS_MIN = 9
 ROWS_MAX = {"plain": 64, "add_norm": 64, "gate_up": 64, "qkv": 64}
 
 
 def _rows_x_ok(x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Tensor], use: str = "") -> bool:
-    """Whether the kernels for more than 16 rows take x with this weight (they read the blocked
+    """Whether the kernels for some tens of rows take x with this weight (they read the blocked
     copy) and, with ``use``, whether they are the faster way for that many rows."""
     return (blocked is not None and x.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-            and x.dim() == 2 and FUSED_MAX_ROWS < x.shape[0] <= ROWS_MAX.get(use, 128) and x.shape[1] % 32 == 0
+            and x.dim() == 2 and ROWS_MIN <= x.shape[0] <= ROWS_MAX.get(use, 128) and x.shape[1] % 32 == 0
             and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
             and w.dim() == 2 and w.shape[1] == x.shape[1])
 
@@ -450,11 +454,11 @@ def gemm_rows_fits(x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Ten
 
 def gemm_rows(x: torch.Tensor, w: torch.Tensor, blocked: torch.Tensor,
               out_dtype: Optional[torch.dtype] = None, splits: int = 1) -> torch.Tensor:
-    """y = x @ w.T for 17 to 128 rows of bfloat16 x, streaming the blocked copy of w once (see
+    """y = x @ w.T for 9 to 128 rows of bfloat16 x, streaming the blocked copy of w once (see
     csrc/gemm_rows.hip). Output bfloat16 or float32 [M, N]; with ``splits`` > 1 the float32
     partial sums [splits, M, N] over that many slices of K (for ``sum_add_rmsnorm``)."""
     if not _rows_x_ok(x, w, blocked):
-        raise KernelError("gemm_rows: needs 17 to 128 rows of bfloat16 x with aligned rows, K a multiple "
+        raise KernelError("gemm_rows: needs 9 to 128 rows of bfloat16 x with aligned rows, K a multiple "
                           "of 32 and the blocked copy of w")
     M, K = x.shape
     N = w.shape[0]
@@ -507,7 +511,7 @@ def gemm_rows_add_rmsnorm_fits(x: torch.Tensor, w: torch.Tensor, blocked: Option
 
 def gemm_rows_add_rmsnorm(x: torch.Tensor, w: torch.Tensor, blocked: torch.Tensor, residual: torch.Tensor,
                           norm_weight: torch.Tensor, eps: float) -> torch.Tensor:
-    """rmsnorm(x @ w.T + residual) * norm_weight for 17 to 128 rows, ``residual`` replaced by the
+    """rmsnorm(x @ w.T + residual) * norm_weight for 9 to 128 rows, ``residual`` replaced by the
     sum: the product as float32 partial sums over slices of K (so that a matrix with few rows
     still gives every compute unit a workgroup), then one kernel that adds them up and
     normalises whole rows."""
@@ -518,27 +522,27 @@ def gemm_rows_add_rmsnorm(x: torch.Tensor, w: torch.Tensor, blocked: torch.Tenso
 
 def gate_up_silu_fits(x: torch.Tensor, w: torch.Tensor, blocked: Optional[torch.Tensor] = None) -> bool:
     """Whether ``gate_up_silu`` is the way to go for x. ``blocked``: the blocked copy of w, which
-    the kernel for more than 16 rows reads."""
-    if _fused_x_ok(x, w):
-        return w.shape[0] % 32 == 0
-    return _rows_x_ok(x, w, blocked, "gate_up") and w.shape[0] % 64 == 0
+    the kernel for some tens of rows reads."""
+    if _rows_x_ok(x, w, blocked, "gate_up") and w.shape[0] % 64 == 0:
+        return True
+    return _fused_x_ok(x, w) and w.shape[0] % 32 == 0
 
 
 def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = None,
                  blocked: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) for w = [Wg; Wu] ([2I, K]) and at most 16 rows of
-    bfloat16 x, in one kernel (see csrc/gemm.hip). ``scale``: the factor that the rows
-    of x still lack; it is applied to both products."""
-    if not ((_fused_x_ok(x, w) and w.shape[0] % 32 == 0) or (_rows_x_ok(x, w, blocked) and w.shape[0] % 64 == 0)):
+    """silu(x Wg^T) * (x Wu^T) for w = [Wg; Wu] ([2I, K]) in one kernel: for at most 16 rows
+    of bfloat16 x the one of csrc/gemm.hip, from ROWS_MIN rows on, with the blocked copy of w,
+    the one of csrc/gemm_rows.hip. ``scale``: the factor that the rows of x still lack (at most
+    16 rows); it is applied to both products."""
+    rows = scale is None and _rows_x_ok(x, w, blocked) and w.shape[0] % 64 == 0
+    if not (rows or (_fused_x_ok(x, w) and w.shape[0] % 32 == 0)):
         raise KernelError("gate_up_silu: needs bfloat16, K a multiple of 8, I a multiple of 16, aligned "
                           "rows, at most 16 of them (up to 128 with the blocked copy of w, K and I "
                           "multiples of 32)")
     M, K = x.shape
     I = w.shape[0] // 2
     out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
-    if M > FUSED_MAX_ROWS:
-        if scale is not None:
-            raise KernelError("gate_up_silu: more than 16 rows come with their factor applied")
+    if rows:
         _check(library.load("gemm_rows").ptl_rows_gate_up_silu(
             _ptr(out), _ptr(x), _rows_weight(w, blocked, "gate_up_silu"), M, I, K,
             ctypes.c_long(x.stride(0)), _stream()), "gate_up_silu")
@@ -556,7 +560,7 @@ def gate_up_silu(x: torch.Tensor, w: torch.Tensor, scale: Optional[RowScale] = N
 def qkv_rope_store_fits(x: torch.Tensor, w: torch.Tensor, head_dim: int,
                         blocked: Optional[torch.Tensor] = None) -> bool:
     """Whether ``qkv_rope_store`` is the way to go for x. ``blocked``: the blocked copy of w, which
-    the kernel for more than 16 rows reads."""
+    the kernel for some tens of rows reads."""
     return (_fused_x_ok(x, w) or _rows_x_ok(x, w, blocked, "qkv")) and head_dim % 32 == 0
 
 
@@ -567,9 +571,11 @@ def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
                    scale: Optional[RowScale] = None, blocked: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q, k, v = x @ w.T (rows of w: q | k | v), q and k rotated, k and v written
     into the cache pages at ``slots``; returns the rotated q [M, Hq, D]. At most 16
-    rows of bfloat16 x, head sizes in steps of 32 (see csrc/gemm.hip). ``scale``: the
-    factor that the rows of x still lack; it is applied to the products."""
-    if not ((_fused_x_ok(x, w) or _rows_x_ok(x, w, blocked)) and head_dim % 32 == 0):
+    rows of bfloat16 x (see csrc/gemm.hip), or, with the blocked copy of w, ROWS_MIN to 128
+    (csrc/gemm_rows.hip); head sizes in steps of 32. ``scale``: the factor that the rows of x
+    still lack (at most 16 rows); it is applied to the products."""
+    rows = scale is None and _rows_x_ok(x, w, blocked)
+    if not ((rows or _fused_x_ok(x, w)) and head_dim % 32 == 0):
         raise KernelError("qkv_rope_store: needs bfloat16, K a multiple of 8, a head size in steps of "
                           "32, aligned rows, at most 16 of them (up to 128 with the blocked copy of w "
                           "and K a multiple of 32)")
@@ -594,9 +600,7 @@ def qkv_rope_store(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor,
                 raise KernelError(f"qkv_rope_store: {name} must be contiguous bfloat16 "
                                   f"[pages, {Hkv}, {page_size}, {D}]")
     q = torch.empty((M, Hq, D), dtype=torch.bfloat16, device=x.device)
-    if M > FUSED_MAX_ROWS:
-        if scale is not None:
-            raise KernelError("qkv_rope_store: more than 16 rows come with their factor applied")
+    if rows:
         # the projection as float32 partial sums over slices of K (few rows of W: so that every
         # compute unit gets a workgroup), then one kernel that adds them up, rotates and stores
         partials = gemm_rows(x, w, blocked, torch.float32, splits=gemm_rows_splits(M, w.shape[0], K))

@@ -32,6 +32,12 @@ class RMSNorm(Part):
 
     def forward(self, x, residual: Optional[torch.Tensor], scale_ok: bool = False):
         if isinstance(x, PendingProduct):
+            # some tens of rows (from ops.ROWS_MIN on): the product as partial sums over slices of
+            # K, then one kernel that adds them up, adds the residual and normalises
+            if (residual is not None and x.blocked is not None
+                    and ops.gemm_rows_add_rmsnorm_fits(x.x, x.w, x.blocked, residual, self.weight)):
+                y = ops.gemm_rows_add_rmsnorm(x.x, x.w, x.blocked, residual, self.weight, self.eps)
+                return y, residual
             # the few rows of a decode step: the product, the residual sum and the weight in one
             # kernel; the rsqrt factor is left to the part that takes the result
             if (scale_ok and residual is not None
@@ -39,12 +45,6 @@ class RMSNorm(Part):
                 y, scale = ops.gemm_skinny_add_norm(x.x, x.w, residual, self.weight, self.eps,
                                                     blocked=x.blocked)
                 return PendingScale(y, scale), residual
-            # some tens of rows: the product as partial sums over slices of K, then one kernel
-            # that adds them up, adds the residual and normalises
-            if (residual is not None and x.blocked is not None
-                    and ops.gemm_rows_add_rmsnorm_fits(x.x, x.w, x.blocked, residual, self.weight)):
-                y = ops.gemm_rows_add_rmsnorm(x.x, x.w, x.blocked, residual, self.weight, self.eps)
-                return y, residual
         x = as_tensor(x)
         y = ops.add_rmsnorm(x, residual, self.weight, self.eps)
         return y, (x if residual is None else residual)

@@ -442,12 +442,14 @@ def test_decode_kernels_read_the_blocked_copy_of_a_weight(ops, dims):
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["to_bf16", "to_fp32"])
 @pytest.mark.parametrize("mnk", [(17, 64, 32), (24, 1000, 96), (33, 2048, 2080), (64, 130, 4096), (100, 3000, 160),
-                                 (128, 16400, 512), (5, 70, 64)])
+                                 (128, 16400, 512), (5, 70, 64), (9, 200, 96), (16, 2048, 2048), (12, 70000, 64),
+                                 (40, 66000, 96)])
 def test_gemm_rows(ops, out_dtype, mnk):
     """The product for some tens of rows (x through LDS, the blocked copy of W streamed): widths
     that are no multiple of a workgroup's 64 rows or of a tile's 16, depths that are no multiple
-    of a chunk, one and two tiles of W a wave, against a float64 product; and as partial sums
-    over slices of K, whose sum is the product."""
+    of a chunk, one to eight tiles of x, one and two tiles of W a wave (two from 1,024 workgroups
+    on), against a float64 product; and as partial sums over slices of K, whose sum is the
+    product."""
     M, N, K = mnk
     torch.manual_seed(21)
     wide = torch.randn(M, K + 8, device="cuda").to(torch.bfloat16)
@@ -456,8 +458,8 @@ def test_gemm_rows(ops, out_dtype, mnk):
     b = ops.blocked_weight(w)
     want = (x.double() @ w.double().T).float()
     t = dict(atol=1e-4, rtol=1e-4) if out_dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
-    y = ops.gemm_rows(x, w, b, out_dtype) if M > 16 else None
-    if M > 16:
+    y = ops.gemm_rows(x, w, b, out_dtype) if M >= ops.ROWS_MIN else None
+    if M >= ops.ROWS_MIN:
         assert y.dtype == out_dtype and y.shape == (M, N)
         torch.testing.assert_close(y.float(), want, **t)
         for splits in (2, 3, 8):
@@ -470,10 +472,11 @@ def test_gemm_rows(ops, out_dtype, mnk):
             ops.gemm_rows(x, w, torch.zeros_like(b)[1:], out_dtype)   # a copy of another matrix
     else:
         with pytest.raises(ops.KernelError):
-            ops.gemm_rows(x, w, b, out_dtype)                      # 16 rows and fewer: the other kernels
+            ops.gemm_rows(x, w, b, out_dtype)                      # fewer rows than ROWS_MIN: the other kernels
 
 
-@pytest.mark.parametrize("mnk", [(17, 64, 96), (40, 2048, 2048), (64, 2056, 320), (128, 4096, 8192)])
+@pytest.mark.parametrize("mnk", [(17, 64, 96), (40, 2048, 2048), (64, 2056, 320), (128, 4096, 8192), (9, 2048, 2048),
+                                 (16, 264, 96)])
 def test_gemm_rows_add_rmsnorm(ops, mnk):
     """Partial sums over slices of K, then one kernel that adds them up, adds the residual and
     normalises whole rows: the residual it leaves and its output are those of the product
@@ -502,7 +505,8 @@ def test_gemm_rows_add_rmsnorm(ops, mnk):
     torch.testing.assert_close(one.float(), got.float(), atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("mik", [(17, 64, 64), (33, 8192, 2048), (64, 352, 160), (128, 1024, 4096)])
+@pytest.mark.parametrize("mik", [(17, 64, 64), (33, 8192, 2048), (64, 352, 160), (128, 1024, 4096), (9, 64, 64),
+                                 (16, 8192, 2048), (13, 352, 160)])
 def test_gate_up_silu_for_tens_of_rows(ops, mik):
     M, I, K = mik
     torch.manual_seed(23)
@@ -512,12 +516,15 @@ def test_gate_up_silu_for_tens_of_rows(ops, mik):
     gu = (x.double() @ w.double().T).float()
     plain = plain_llama.silu(gu[:, :I]) * gu[:, I:]
     torch.testing.assert_close(got.float(), plain, atol=3e-2, rtol=3e-2)
-    with pytest.raises(ops.KernelError):
-        ops.gate_up_silu(x, w)                                           # no blocked copy: not this many rows
+    if M > 16:
+        with pytest.raises(ops.KernelError):
+            ops.gate_up_silu(x, w)                                       # no blocked copy: not this many rows
+    else:                                                                # the kernel for at most 16 rows
+        torch.testing.assert_close(ops.gate_up_silu(x, w).float(), plain, atol=3e-2, rtol=3e-2)
 
 
 @pytest.mark.parametrize("dims", [(4, 2, 64, 16, 96, 20), (3, 1, 32, 4, 128, 33), (32, 8, 128, 16, 4096, 64),
-                                  (6, 3, 96, 8, 224, 128)])
+                                  (6, 3, 96, 8, 224, 128), (32, 8, 64, 16, 2048, 9), (5, 5, 32, 2, 160, 16)])
 def test_qkv_rope_store_for_tens_of_rows(ops, dims):
     """Partial sums of the projection, then one kernel that adds them up, rotates q and k and
     writes k and v into their pages, against the plain formulas; rows whose slot is -1 store
