@@ -42,13 +42,14 @@ enum { MODE_PLAIN = 0, MODE_SILU = 1 };
 
 constexpr int TILES = 4;                   // tiles of 16 weight rows a workgroup owns: 64 rows
 constexpr int NB = 3;                      // chunks of x in LDS: one in use, two on their way
-// Columns of a chunk (KC) and chunks of W a wave has under way (DEPTH) for 1, 2, 4 and 8 tiles of
+// Columns of a chunk (KC) and chunks of W a wave has under way (DEPTH) for 1, 2, 3, 4 and 8 tiles of
 // x, with one tile of W a wave: 8 KB of weights a wave in flight, chunks of x of at most 32 KB.
 // Measured at 64 rows and the 1B widths: 128 to 512 columns a chunk and 2 to 12 chunks under
 // way differ by a few per cent. With two tiles a wave: 128 columns, 4 chunks (the head of
 // vocabulary size: 112 us against 137 with 256 and 2).
 constexpr int KC_1 = 256, DEPTH_1 = 2;
 constexpr int KC_2 = 256, DEPTH_2 = 2;
+constexpr int KC_3 = 256, DEPTH_3 = 2;
 constexpr int KC_4 = 256, DEPTH_4 = 2;
 constexpr int KC_8 = 128, DEPTH_8 = 4;
 
@@ -341,7 +342,7 @@ bool bad_common(int M, int K, long ldx) {
   return M <= 0 || M > 128 || K <= 0 || K % 32 || ldx % 8 || ldx < K;
 }
 
-int m_tiles(int M) { return M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8; }
+int m_tiles(int M) { return M <= 16 ? 1 : M <= 32 ? 2 : M <= 48 ? 3 : M <= 64 ? 4 : 8; }
 
 // The slices of K that a product should be cut into when the caller can take partial sums:
 // doubled while the workgroups are fewer than the compute units and a slice keeps at least 256
@@ -383,6 +384,7 @@ extern "C" int ptl_rows_gemm_bf16(void* y, const void* x, const void* w_blocked,
   switch (m_tiles(M)) {
     case 1: return BY_WT(1, KC_1, DEPTH_1);
     case 2: return BY_WT(2, KC_2, DEPTH_2);
+    case 3: return BY_WT(3, KC_3, DEPTH_3);
     case 4: return BY_WT(4, KC_4, DEPTH_4);
     default: return BY_WT(8, KC_8, DEPTH_8);
   }
@@ -402,6 +404,7 @@ extern "C" int ptl_rows_gate_up_silu(void* out, const void* x, const void* w_blo
   switch (m_tiles(M)) {
     case 1: return GO(1, KC_1, DEPTH_1);
     case 2: return GO(2, KC_2, DEPTH_2);
+    case 3: return GO(3, KC_3, DEPTH_3);
     case 4: return GO(4, KC_4, DEPTH_4);
     default: return GO(8, KC_8, DEPTH_8);
   }

@@ -42,10 +42,13 @@ from .batch import SeqInput, StepEntry, StepLayout, StepSizes, take_pages
 
 
 def bucket_sizes(max_num_seqs: int) -> List[int]:
+    """Numbers of decoding rows that steps are padded to: powers of two up to 32, then every 16
+    (a tile of rows of the decode products: 33 to 48 rows cost less than 49 to 64), and the
+    most the engine admits."""
     out, b = [], 1
     while b < max_num_seqs:
         out.append(b)
-        b *= 2
+        b = b * 2 if b < 32 else b + 16
     out.append(max_num_seqs)
     return out
 

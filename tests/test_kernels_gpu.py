@@ -443,7 +443,7 @@ def test_decode_kernels_read_the_blocked_copy_of_a_weight(ops, dims):
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["to_bf16", "to_fp32"])
 @pytest.mark.parametrize("mnk", [(17, 64, 32), (24, 1000, 96), (33, 2048, 2080), (64, 130, 4096), (100, 3000, 160),
                                  (128, 16400, 512), (5, 70, 64), (9, 200, 96), (16, 2048, 2048), (12, 70000, 64),
-                                 (40, 66000, 96)])
+                                 (40, 66000, 96), (48, 3072, 2048), (37, 100, 4128)])
 def test_gemm_rows(ops, out_dtype, mnk):
     """The product for some tens of rows (x through LDS, the blocked copy of W streamed): widths
     that are no multiple of a workgroup's 64 rows or of a tile's 16, depths that are no multiple
@@ -476,7 +476,7 @@ def test_gemm_rows(ops, out_dtype, mnk):
 
 
 @pytest.mark.parametrize("mnk", [(17, 64, 96), (40, 2048, 2048), (64, 2056, 320), (128, 4096, 8192), (9, 2048, 2048),
-                                 (16, 264, 96)])
+                                 (16, 264, 96), (48, 2048, 8192), (35, 72, 64)])
 def test_gemm_rows_add_rmsnorm(ops, mnk):
     """Partial sums over slices of K, then one kernel that adds them up, adds the residual and
     normalises whole rows: the residual it leaves and its output are those of the product
@@ -506,7 +506,7 @@ def test_gemm_rows_add_rmsnorm(ops, mnk):
 
 
 @pytest.mark.parametrize("mik", [(17, 64, 64), (33, 8192, 2048), (64, 352, 160), (128, 1024, 4096), (9, 64, 64),
-                                 (16, 8192, 2048), (13, 352, 160)])
+                                 (16, 8192, 2048), (13, 352, 160), (44, 2048, 512), (48, 96, 64)])
 def test_gate_up_silu_for_tens_of_rows(ops, mik):
     M, I, K = mik
     torch.manual_seed(23)
@@ -524,7 +524,8 @@ def test_gate_up_silu_for_tens_of_rows(ops, mik):
 
 
 @pytest.mark.parametrize("dims", [(4, 2, 64, 16, 96, 20), (3, 1, 32, 4, 128, 33), (32, 8, 128, 16, 4096, 64),
-                                  (6, 3, 96, 8, 224, 128), (32, 8, 64, 16, 2048, 9), (5, 5, 32, 2, 160, 16)])
+                                  (6, 3, 96, 8, 224, 128), (32, 8, 64, 16, 2048, 9), (5, 5, 32, 2, 160, 16),
+                                  (8, 2, 64, 16, 512, 48), (3, 3, 96, 4, 96, 37)])
 def test_qkv_rope_store_for_tens_of_rows(ops, dims):
     """Partial sums of the projection, then one kernel that adds them up, rotates q and k and
     writes k and v into their pages, against the plain formulas; rows whose slot is -1 store
