@@ -42,12 +42,15 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     to_f32 = out_dtype == torch.float32
     # measured on MI355X at the 1B shapes: the weight-streaming kernel is level with the
     # library up to 8 rows (and ahead for the vocabulary-sized head); beyond that the library
-    if (M <= SKINNY_ROWS or (to_f32 and M <= SKINNY_ROWS_F32)) and ops.gemm_skinny_fits(x, w):
+    if M <= SKINNY_ROWS and ops.gemm_skinny_fits(x, w):
         return ops.gemm_skinny(x, w, out_dtype, blocked=blocked)
-    # some tens of rows (a large decoding batch): the kernel that streams the blocked copy with
-    # x staged through LDS, where measured faster than the library
+    # some tens of rows (a large decoding batch, from ops.ROWS_MIN rows on): the kernel that
+    # streams the blocked copy with x staged through LDS, where measured faster than the library
+    # (and, for a vocabulary-sized head of 9 to 16 rows, than the skinny kernel)
     if ops.gemm_rows_fits(x, w, blocked):
         return ops.gemm_rows(x, w, blocked, out_dtype)
+    if to_f32 and M <= SKINNY_ROWS_F32 and ops.gemm_skinny_fits(x, w):
+        return ops.gemm_skinny(x, w, out_dtype, blocked=blocked)
     if ops.gemm_library_fits(x, w):
         return ops.gemm_library(x, w, out_dtype, checked=True)
     if to_f32:
